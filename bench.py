@@ -1,0 +1,265 @@
+#!/usr/bin/env python3
+"""Benchmark of the dispatch-layout + permute + combine path on one MI355X.
+
+One step = one pass of the three kernels over one batch of synthetic input that already sits
+in HBM: fused layout -> permute into the expert-contiguous buffer -> weighted combine of fresh
+bf16 expert outputs.  Prints one JSON line (see the keys below).  The CPU checker is timed on a
+bounded sample of the same workload as a reported baseline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config target|c2|c3|c4|c5]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBPS = 8000.0      # MI355X published HBM3E bandwidth
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="target")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    return ap.parse_args()
+
+
+class Workload:
+    """Device buffers and raw C-ABI calls of one configuration (nothing allocates in a step)."""
+
+    def __init__(self, cfg, dev):
+        import numpy as np
+        import torch
+        from commbench_amd import _lib, workloads as wl
+
+        self.cfg, self.torch, self.lib, self._lib = cfg, torch, _lib.load(), _lib
+        T, K, E, R, H = cfg.num_tokens, cfg.num_topk, cfg.num_experts, cfg.num_ranks, cfg.hidden
+        topk_np, w_np = wl.make_routing(cfg)
+        self.topk_np, self.w_np = topk_np, w_np
+        self.num_routes = int((topk_np >= 0).sum())
+        self.topk = torch.from_numpy(topk_np).to(dev)
+        self.w = torch.from_numpy(w_np).to(dev)
+        gen = torch.Generator(device=dev).manual_seed(wl.SEED_BASE + cfg.config_id)
+        x = torch.randn((T, H), device=dev, generator=gen, dtype=torch.float32).to(torch.bfloat16)
+        self.scales = None
+        if cfg.payload == "fp8":
+            xf = x.to(torch.float32).view(T, H // 128, 128)
+            amax = xf.abs().amax(dim=2)
+            self.scales = torch.where(amax > 0, amax / 448.0, torch.ones_like(amax)).contiguous()
+            x = (xf / self.scales[:, :, None]).clamp_(-448, 448).to(torch.float8_e4m3fn).view(T, H)
+        self.x = x.contiguous()
+        cap = T * K
+        self.cap = cap
+        self.recv_x = torch.empty((cap, H), dtype=self.x.dtype, device=dev)
+        self.recv_scales = (torch.empty((cap, cfg.num_scales), dtype=torch.float32, device=dev)
+                            if self.scales is not None else None)
+        # Expert outputs: a buffer of their own, so combine reads from HBM, not from lines the
+        # permute just wrote.
+        self.y = torch.empty((cap, H), dtype=torch.bfloat16, device=dev)
+        for i in range(0, cap, 8192):
+            n = min(8192, cap - i)
+            self.y[i:i + n] = torch.randn((n, H), device=dev, generator=gen).to(torch.bfloat16)
+        i32 = dict(dtype=torch.int32, device=dev)
+        self.per_rank = torch.empty(R, **i32)
+        self.per_expert = torch.empty(E, **i32)
+        self.in_rank = torch.empty((T, R), dtype=torch.bool, device=dev)
+        self.off = torch.empty(E + 1, **i32)
+        self.psum = torch.empty(R, **i32)
+        self.slot_rel = torch.empty((T, K), **i32)
+        self.slot_map = torch.empty((T, K), **i32)
+        self.src_map = torch.empty(cap, **i32)
+        self.recv_idx = torch.empty(cap, dtype=torch.int64, device=dev)
+        self.recv_w = torch.empty(cap, dtype=torch.float32, device=dev)
+        self.out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+        ws_bytes = self.lib.mi_ep_workspace_bytes(T, K, E, R)
+        self.ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        self.stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(self.lib.mi_ep_workspace_init(self.ws.data_ptr(), ws_bytes, self.stream), "ws init")
+        self.bytes = wl.algorithmic_bytes(T, H, E, K, R, self.num_routes,
+                                          1 if cfg.payload == "fp8" else 2, cfg.num_scales)
+
+    def layout(self):
+        c = self.cfg
+        self._lib.check(self.lib.mi_ep_dispatch_layout(
+            self.topk.data_ptr(), c.num_tokens, c.num_topk, c.num_ranks, c.num_experts, 1, 0,
+            self.per_rank.data_ptr(), self.per_expert.data_ptr(), self.in_rank.data_ptr(),
+            self.off.data_ptr(), self.psum.data_ptr(), None, self.slot_rel.data_ptr(),
+            self.ws.data_ptr(), self.ws.numel(), self.stream), "layout")
+
+    def dispatch(self):
+        c = self.cfg
+        self._lib.check(self.lib.mi_ep_dispatch(
+            self.x.data_ptr(), None if self.scales is None else self.scales.data_ptr(),
+            self.topk.data_ptr(), self.w.data_ptr(), self.off.data_ptr(), self.slot_rel.data_ptr(),
+            self.per_expert.data_ptr(), c.num_tokens, c.num_topk, c.num_experts, 1, c.row_bytes,
+            c.num_scales, self.recv_x.data_ptr(),
+            None if self.recv_scales is None else self.recv_scales.data_ptr(),
+            self.src_map.data_ptr(), self.recv_idx.data_ptr(), self.recv_w.data_ptr(),
+            self.slot_map.data_ptr(), self.cap, self.stream), "dispatch")
+
+    def combine(self):
+        c = self.cfg
+        self._lib.check(self.lib.mi_ep_combine(
+            self.y.data_ptr(), self.slot_map.data_ptr(), self.w.data_ptr(), None, None, None,
+            c.num_tokens, c.num_topk, c.hidden, self.out.data_ptr(), None, self.stream), "combine")
+
+    def step(self):
+        self.layout()
+        self.dispatch()
+        self.combine()
+
+
+def cpu_baseline(cfg, seconds):
+    """The CPU checker on a bounded token sample of the same workload, one thread and all the
+    host cores this job may use; returns the cpu_baseline object."""
+    import numpy as np
+    from commbench_amd import workloads as wl
+    from oracle import ep_oracle
+
+    sample_tokens = min(cfg.num_tokens, 1024)
+    topk_np, w_np = wl.make_routing(cfg)
+    topk_np, w_np = topk_np[:sample_tokens].copy(), w_np[:sample_tokens].copy()
+    rng = np.random.Generator(np.random.PCG64(1))
+    x = rng.integers(0, 1 << 16, size=(sample_tokens, cfg.row_bytes // 2), dtype=np.uint16)
+    scales = (rng.standard_normal((sample_tokens, cfg.num_scales)).astype(np.float32)
+              if cfg.num_scales else None)
+    rows = int((topk_np >= 0).sum())
+    y = ep_oracle.f32_to_bf16(rng.standard_normal((rows, cfg.hidden), dtype=np.float32))
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    threads = max(1, min(threads, os.cpu_count() or 1, 16))
+
+    def one_pass(nthreads):
+        res = ep_oracle.full_path(topk_np, w_np, x.view(np.uint8), scales, cfg.num_experts,
+                                  cfg.num_ranks, 1, nthreads)
+        ep_oracle.combine(y, res["slot_map"], w_np, num_threads=nthreads)
+
+    def rate(nthreads, budget):
+        one_pass(nthreads)                           # warm
+        n, t0 = 0, time.perf_counter()
+        while True:
+            one_pass(nthreads)
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt >= budget:
+                return n * sample_tokens / dt
+
+    single = rate(1, seconds * 0.5)
+    multi = rate(threads, seconds * 0.5) if threads > 1 else single
+    return {"value": multi, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "single_thread_value": single,
+            "sample": f"first {sample_tokens} tokens of the workload ({rows} routes): layout + "
+                      f"offsets + slot maps + permute + combine, repeated for ~{seconds:.0f} s "
+                      f"(half on 1 thread, half on {threads} OpenMP threads)"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported "
+              "(this path has no multi-GPU leg; partitions of one GPU's HBM stand for ranks)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from commbench_amd import workloads as wl
+
+    cfg = wl.CONFIGS[args.config]
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    wk = Workload(cfg, dev)
+    T = cfg.num_tokens
+
+    for _ in range(args.warmup):
+        wk.step()
+    torch.cuda.synchronize()
+
+    # Timed region: exactly `steps` steps; HIP events on the launch stream bracket each kernel.
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for ev in marks:
+        ev[0].record()
+        wk.layout()
+        ev[1].record()
+        wk.dispatch()
+        ev[2].record()
+        wk.combine()
+        ev[3].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    names = ["ep_layout_fused_kernel", "ep_permute_kernel", "ep_combine_kernel"]
+    kernel_us = {n: sum(ev[i].elapsed_time(ev[i + 1]) for ev in marks) * 1e3 / args.steps
+                 for i, n in enumerate(names)}
+    kernel_bytes = dict(zip(names, (wk.bytes["layout"], wk.bytes["dispatch"], wk.bytes["combine"])))
+    dominant = max(names, key=lambda n: kernel_us[n])
+    achieved = kernel_bytes[dominant] / (kernel_us[dominant] * 1e-6) / 1e9
+
+    # Measured streaming-copy ceiling next to the nominal peak (read + write of 1 GiB).
+    from commbench_amd import ops
+    src = wk.y.view(torch.uint8).reshape(-1)[: 1 << 30]
+    dst = wk.recv_x.view(torch.uint8).reshape(-1)[: src.numel()]
+    src = src[: dst.numel()]
+    for _ in range(3):
+        ops.copy_yardstick(dst, src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        ops.copy_yardstick(dst, src)
+    e1.record()
+    torch.cuda.synchronize()
+    copy_gbps = 2 * src.numel() * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+    traffic = None
+    traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as f:
+            traffic = json.load(f).get(cfg.name, {}).get(dominant)
+
+    result = {
+        "metric": "dispatch+combine tokens/s and achieved HBM GB/s (% of peak), 1 MI355X",
+        "value": T / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if cfg.payload == "bf16" else "u8",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{cfg.name}: layout + permute + combine, {T} tokens x {cfg.hidden} hidden "
+                        f"{cfg.payload}, {cfg.num_experts} experts, top-{cfg.num_topk}, "
+                        f"{cfg.num_ranks} HBM partitions, {cfg.routing} routing, "
+                        f"{wk.num_routes} routes",
+            "num_tokens": T, "hidden": cfg.hidden, "num_experts": cfg.num_experts,
+            "num_topk": cfg.num_topk, "num_ranks": cfg.num_ranks, "payload": cfg.payload,
+        },
+        "hbm_gbps_whole_step": wk.bytes["total"] / (ms_per_step * 1e-3) / 1e9,
+        "hbm_frac_whole_step": wk.bytes["total"] / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+        "algorithmic_bytes": wk.bytes,
+        "kernel_us": kernel_us,
+        "kernel_gbps": {n: kernel_bytes[n] / (kernel_us[n] * 1e-6) / 1e9 for n in names},
+        "copy_yardstick_gbps": copy_gbps,
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
+                     "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBPS,
+                     "traffic": traffic},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,230 @@
+// extern "C" boundary of the gfx950 dispatch core: argument checks on the host,
+// then kernel launches.  No allocation, no synchronisation (except
+// mi_ep_workspace_status, which says so), no process-wide state.
+#include "../../include/mi_ep.h"
+
+#include "ep_device.h"
+
+namespace {
+
+using namespace mi_ep;
+
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// The reference's constructor checks (example042 .cu:96-107) plus the limits of
+// these kernels.
+inline bool routing_shape_ok(int num_tokens, int num_topk, int num_ranks, int num_experts) {
+  if (num_tokens < 0) return false;
+  if (num_ranks <= 0 || num_ranks > MI_EP_MAX_RANKS) return false;
+  if (num_topk <= 0 || num_topk > MI_EP_MAX_TOPK) return false;
+  if (num_experts <= 0 || num_experts > MI_EP_MAX_EXPERTS) return false;
+  if (num_experts % num_ranks != 0) return false;
+  if (static_cast<long long>(num_tokens) * num_topk >= (1LL << 30)) return false;
+  return true;
+}
+
+inline int num_tiles_for(int num_tokens) { return (num_tokens + kTileTokens - 1) / kTileTokens; }
+
+inline int status_of(hipError_t e) { return e == hipSuccess ? MI_EP_OK : static_cast<int>(e); }
+
+// Bounded device-side wait: polls spaced by s_sleep, roughly a microsecond apart,
+// so a few seconds before a launch gives up and flags the workspace.
+constexpr uint32_t kSpinLimit = 1u << 22;
+
+}  // namespace
+
+extern "C" {
+
+int mi_ep_abi_version(void) { return MI_EP_ABI_VERSION; }
+
+const char* mi_ep_strerror(int code) {
+  switch (code) {
+    case MI_EP_OK: return "ok";
+    case MI_EP_EINVAL: return "invalid argument";
+    case MI_EP_ENOSPC: return "workspace too small";
+    case MI_EP_ETIMEDOUT: return "device-side wait timed out";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+  return "unknown error";
+}
+
+int mi_ep_get_dispatch_layout(const int64_t* topk_idx, int* num_tokens_per_rank,
+                              int* num_tokens_per_rdma_rank, int* num_tokens_per_expert,
+                              bool* is_token_in_rank, int num_tokens, int num_topk, int num_ranks,
+                              int num_experts, void* stream) {
+  (void)num_tokens_per_rdma_rank;
+  if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
+  if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
+  if (num_tokens > 0 && (topk_idx == nullptr || is_token_in_rank == nullptr)) return MI_EP_EINVAL;
+  return status_of(launch_layout_counts(topk_idx, num_tokens_per_rank, num_tokens_per_expert,
+                                        reinterpret_cast<uint8_t*>(is_token_in_rank), num_tokens,
+                                        num_topk, num_ranks, num_experts, as_stream(stream)));
+}
+
+size_t mi_ep_workspace_bytes(int num_tokens, int num_topk, int num_experts, int num_ranks) {
+  if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return 0;
+  const size_t tiles = static_cast<size_t>(num_tiles_for(num_tokens));
+  return sizeof(LayoutWorkspace) + tiles * static_cast<size_t>(num_experts + num_ranks) * sizeof(uint64_t);
+}
+
+int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+  if (workspace == nullptr || workspace_bytes < sizeof(LayoutWorkspace)) return MI_EP_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
+  return status_of(launch_fill_u32(static_cast<uint32_t*>(workspace), workspace_bytes / 4, 0u,
+                                   as_stream(stream)));
+}
+
+int mi_ep_workspace_status(const void* workspace, void* stream) {
+  if (workspace == nullptr) return MI_EP_EINVAL;
+  LayoutWorkspace header;
+  hipError_t e = hipMemcpyAsync(&header, workspace, sizeof(uint32_t) * 4, hipMemcpyDeviceToHost,
+                                as_stream(stream));
+  if (e != hipSuccess) return static_cast<int>(e);
+  e = hipStreamSynchronize(as_stream(stream));
+  if (e != hipSuccess) return static_cast<int>(e);
+  return header.timed_out != 0 ? MI_EP_ETIMEDOUT : MI_EP_OK;
+}
+
+int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
+                          int num_experts, int expert_alignment, int num_channels,
+                          int* num_tokens_per_rank, int* num_tokens_per_expert,
+                          bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
+                          int* channel_prefix_matrix, int* slot_rel, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
+  if (expert_alignment < 1) return MI_EP_EINVAL;
+  if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
+  if (channel_prefix_matrix != nullptr && (num_channels < 1 || num_channels > 4096)) return MI_EP_EINVAL;
+  if (psum_rank_rows != nullptr && expert_offsets == nullptr) return MI_EP_EINVAL;
+  // Padded totals must stay inside int32.
+  if ((static_cast<long long>(num_tokens) * num_topk +
+       static_cast<long long>(num_experts) * (expert_alignment - 1)) >= (1LL << 31))
+    return MI_EP_EINVAL;
+  hipStream_t s = as_stream(stream);
+
+  if (num_tokens == 0) {
+    // Nothing to scan: every output is zero.
+    hipError_t e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_rank), num_ranks, 0u, s);
+    if (e == hipSuccess)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_expert), num_experts, 0u, s);
+    if (e == hipSuccess && expert_offsets != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(expert_offsets), num_experts + 1, 0u, s);
+    if (e == hipSuccess && psum_rank_rows != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(psum_rank_rows), num_ranks, 0u, s);
+    if (e == hipSuccess && channel_prefix_matrix != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(channel_prefix_matrix),
+                          static_cast<size_t>(num_ranks) * num_channels, 0u, s);
+    return status_of(e);
+  }
+
+  if (topk_idx == nullptr || is_token_in_rank == nullptr || workspace == nullptr) return MI_EP_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
+  if (workspace_bytes < mi_ep_workspace_bytes(num_tokens, num_topk, num_experts, num_ranks))
+    return MI_EP_ENOSPC;
+
+  LayoutArgs a{};
+  a.topk_idx = topk_idx;
+  a.num_tokens_per_rank = num_tokens_per_rank;
+  a.num_tokens_per_expert = num_tokens_per_expert;
+  a.is_token_in_rank = reinterpret_cast<uint8_t*>(is_token_in_rank);
+  a.expert_offsets = expert_offsets;
+  a.psum_rank_rows = psum_rank_rows;
+  a.channel_prefix_matrix = channel_prefix_matrix;
+  a.slot_rel = slot_rel;
+  a.ws = static_cast<LayoutWorkspace*>(workspace);
+  a.num_tokens = num_tokens;
+  a.num_topk = num_topk;
+  a.num_ranks = num_ranks;
+  a.num_experts = num_experts;
+  a.experts_per_rank = num_experts / num_ranks;
+  a.expert_alignment = expert_alignment;
+  a.num_channels = num_channels;
+  a.num_tiles = num_tiles_for(num_tokens);
+  a.expert_bits = 1;
+  while ((1 << a.expert_bits) < num_experts) ++a.expert_bits;
+  a.spin_limit = kSpinLimit;
+  return status_of(launch_layout_fused(a, s));
+}
+
+int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
+                   const float* topk_weights, const int* expert_offsets, const int* slot_rel,
+                   const int* num_tokens_per_expert, int num_tokens, int num_topk,
+                   int num_experts, int expert_alignment, int row_bytes, int num_scales,
+                   void* recv_x, float* recv_scales, int* recv_src_map, int64_t* recv_topk_idx,
+                   float* recv_topk_weights, int* slot_map, int capacity_rows, void* stream) {
+  if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK) return MI_EP_EINVAL;
+  if (num_experts <= 0 || num_experts > MI_EP_MAX_EXPERTS || expert_alignment < 1) return MI_EP_EINVAL;
+  if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
+  if (expert_offsets == nullptr || recv_src_map == nullptr) return MI_EP_EINVAL;
+  if (capacity_rows > 0 && recv_x == nullptr) return MI_EP_EINVAL;
+  if (!aligned16(x) || !aligned16(recv_x)) return MI_EP_EINVAL;
+  if (num_tokens > 0 &&
+      (x == nullptr || topk_idx == nullptr || slot_rel == nullptr || slot_map == nullptr))
+    return MI_EP_EINVAL;
+  if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
+  if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
+  if (expert_alignment > 1 && num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
+
+  PermuteArgs a{};
+  a.x = static_cast<const vec16*>(x);
+  a.x_scales = x_scales;
+  a.topk_idx = topk_idx;
+  a.topk_weights = topk_weights;
+  a.expert_offsets = expert_offsets;
+  a.slot_rel = slot_rel;
+  a.num_tokens_per_expert = num_tokens_per_expert;
+  a.recv_x = static_cast<vec16*>(recv_x);
+  a.recv_scales = recv_scales;
+  a.recv_src_map = recv_src_map;
+  a.recv_topk_idx = recv_topk_idx;
+  a.recv_topk_weights = recv_topk_weights;
+  a.slot_map = slot_map;
+  a.num_tokens = num_tokens;
+  a.num_topk = num_topk;
+  a.num_experts = num_experts;
+  a.row_vecs = row_bytes / 16;
+  a.num_scales = num_scales;
+  a.capacity_rows = capacity_rows;
+  hipStream_t s = as_stream(stream);
+  hipError_t e = launch_permute(a, s);
+  if (e == hipSuccess && expert_alignment > 1) e = launch_pad_rows(a, s);
+  return status_of(e);
+}
+
+int mi_ep_combine(const void* y, const int* slot_map, const float* topk_weights,
+                  const void* bias_0, const void* bias_1, const float* recv_topk_weights,
+                  int num_tokens, int num_topk, int hidden, void* combined_x,
+                  float* combined_topk_weights, void* stream) {
+  if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK) return MI_EP_EINVAL;
+  if (hidden <= 0 || hidden % 8 != 0) return MI_EP_EINVAL;
+  if ((recv_topk_weights != nullptr) != (combined_topk_weights != nullptr)) return MI_EP_EINVAL;
+  if (num_tokens > 0 && (slot_map == nullptr || combined_x == nullptr)) return MI_EP_EINVAL;
+  if (!aligned16(y) || !aligned16(bias_0) || !aligned16(bias_1) || !aligned16(combined_x))
+    return MI_EP_EINVAL;
+
+  CombineArgs a{};
+  a.y = static_cast<const vec16*>(y);
+  a.slot_map = slot_map;
+  a.topk_weights = topk_weights;
+  a.bias_0 = static_cast<const vec16*>(bias_0);
+  a.bias_1 = static_cast<const vec16*>(bias_1);
+  a.recv_topk_weights = recv_topk_weights;
+  a.combined_x = static_cast<vec16*>(combined_x);
+  a.combined_topk_weights = combined_topk_weights;
+  a.num_tokens = num_tokens;
+  a.num_topk = num_topk;
+  a.row_vecs = hidden / 8;
+  return status_of(launch_combine(a, as_stream(stream)));
+}
+
+int mi_ep_copy_yardstick(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes % 16 != 0 || !aligned16(dst) || !aligned16(src)) return MI_EP_EINVAL;
+  if (bytes > 0 && (dst == nullptr || src == nullptr)) return MI_EP_EINVAL;
+  return status_of(launch_copy_yardstick(static_cast<vec16*>(dst), static_cast<const vec16*>(src),
+                                         bytes / 16, as_stream(stream)));
+}
+
+}  // extern "C"

@@ -1,0 +1,134 @@
+// Shared device helpers and launcher declarations for the gfx950 dispatch core.
+// Wave64 only: every kernel here assumes 64-lane wavefronts.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi_ep {
+
+// 16 bytes as a native vector, so that non-temporal builtins accept it.
+typedef uint32_t vec16 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+constexpr int kMaxRanks = 8;
+constexpr int kMaxTopk = 8;
+constexpr int kMaxExperts = 1024;
+
+// ---- layout ---------------------------------------------------------------
+constexpr int kLayoutThreads = 256;
+constexpr int kLayoutWaves = kLayoutThreads / kWave;
+constexpr int kTileTokens = 256;  // one token per thread of the tile's workgroup
+
+// Header of the fused layout kernel's workspace; the look-back status words follow.
+struct alignas(256) LayoutWorkspace {
+  uint32_t ticket;      // next tile to hand out
+  uint32_t done;        // tiles finished in the running launch
+  uint32_t generation;  // bumped by the last tile of every launch
+  uint32_t timed_out;   // sticky: a bounded wait expired
+};
+
+struct LayoutArgs {
+  const int64_t* topk_idx;
+  int* num_tokens_per_rank;
+  int* num_tokens_per_expert;
+  uint8_t* is_token_in_rank;
+  int* expert_offsets;
+  int* psum_rank_rows;
+  int* channel_prefix_matrix;
+  int* slot_rel;
+  LayoutWorkspace* ws;
+  int num_tokens;
+  int num_topk;
+  int num_ranks;
+  int num_experts;
+  int experts_per_rank;
+  int expert_alignment;
+  int num_channels;
+  int num_tiles;
+  int expert_bits;  // ceil(log2(num_experts)), at least 1
+  uint32_t spin_limit;
+};
+
+hipError_t launch_layout_fused(const LayoutArgs& a, hipStream_t stream);
+hipError_t launch_layout_counts(const int64_t* topk_idx, int* num_tokens_per_rank,
+                                int* num_tokens_per_expert, uint8_t* is_token_in_rank,
+                                int num_tokens, int num_topk, int num_ranks, int num_experts,
+                                hipStream_t stream);
+hipError_t launch_fill_u32(uint32_t* dst, size_t count, uint32_t value, hipStream_t stream);
+
+// ---- permute ----------------------------------------------------------------
+struct PermuteArgs {
+  const vec16* x;
+  const float* x_scales;
+  const int64_t* topk_idx;
+  const float* topk_weights;
+  const int* expert_offsets;
+  const int* slot_rel;
+  const int* num_tokens_per_expert;
+  vec16* recv_x;
+  float* recv_scales;
+  int* recv_src_map;
+  int64_t* recv_topk_idx;
+  float* recv_topk_weights;
+  int* slot_map;
+  int num_tokens;
+  int num_topk;
+  int num_experts;
+  int row_vecs;  // 16-byte vectors per row
+  int num_scales;
+  int capacity_rows;
+};
+
+hipError_t launch_permute(const PermuteArgs& a, hipStream_t stream);
+hipError_t launch_pad_rows(const PermuteArgs& a, hipStream_t stream);
+
+// ---- combine ----------------------------------------------------------------
+struct CombineArgs {
+  const vec16* y;
+  const int* slot_map;
+  const float* topk_weights;
+  const vec16* bias_0;
+  const vec16* bias_1;
+  const float* recv_topk_weights;
+  vec16* combined_x;
+  float* combined_topk_weights;
+  int num_tokens;
+  int num_topk;
+  int row_vecs;  // 16-byte vectors (8 bf16) per row
+};
+
+hipError_t launch_combine(const CombineArgs& a, hipStream_t stream);
+
+hipError_t launch_copy_yardstick(vec16* dst, const vec16* src, size_t vecs, hipStream_t stream);
+
+// ---- device helpers -------------------------------------------------------
+#ifdef __HIPCC__
+__device__ __forceinline__ int lane_id() { return static_cast<int>(threadIdx.x) & (kWave - 1); }
+
+__device__ __forceinline__ uint64_t lanes_below(int lane) { return (1ull << lane) - 1ull; }
+
+// Value of `v` in lane `src` (wave-uniform src), as a scalar.
+__device__ __forceinline__ int wave_read(int v, int src) {
+  return __builtin_amdgcn_readlane(v, src);
+}
+__device__ __forceinline__ float wave_read(float v, int src) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// fp32 -> bf16 bits, round to nearest even, NaN kept quiet.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  uint32_t nan = (u >> 16) | 0x0040u;
+  return ((u & 0x7fffffffu) > 0x7f800000u) ? nan : rounded;
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (f32_to_bf16_bits(lo) & 0xffffu) | (f32_to_bf16_bits(hi) << 16);
+}
+#endif
+
+}  // namespace mi_ep

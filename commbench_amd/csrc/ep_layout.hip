@@ -1,0 +1,401 @@
+// Layout kernels for gfx950.
+//
+// ep_layout_fused_kernel: one pass over topk_idx that yields per-expert counts,
+// de-duplicated per-rank counts, is_token_in_rank, aligned exclusive expert
+// offsets, inclusive per-partition rows, per-channel inclusive prefixes and the
+// deterministic position of every route inside its expert segment.  It replaces
+// the reference's layout kernel (example042 .cu:48-86), the notify role of
+// dispatch_impl (example080 .cu:78-240), the deterministic prologue
+// (example078 .cu:27-43) and the channel half of notify_dispatch
+// (example047 .cu:132-143).
+//
+// Shape of the computation (wave64):
+//   * a tile is 256 tokens = 256*K routes, owned by one 256-thread workgroup;
+//     tiles are handed out by an atomic ticket so that every tile's predecessors
+//     have already started, which makes the look-back below deadlock-free
+//     whatever the residency of the grid;
+//   * each wave walks its 64*K routes in 64-route chunks in (token, slot) order;
+//     lanes holding the same expert find each other with log2(E) ballots, the
+//     lowest such lane bumps the wave's private LDS counter once, and every lane
+//     derives its rank among equals with a popcount -- no LDS atomics, so routing
+//     skew costs nothing;
+//   * columns (E experts followed by R ranks) are scanned across tiles with a
+//     single-pass decoupled look-back on 64-bit status words
+//     {flag:2 | generation:30 | value:32}; the generation tag makes the words of
+//     earlier launches invalid without any clearing pass;
+//   * the tile holding the last ticket knows every column total and emits counts
+//     and the aligned offsets.
+//
+// ep_layout_counts_kernel: the workspace-free variant behind the reference's
+// DeepepDispatchLayout::compute signature (counts and flags only).
+#include "ep_device.h"
+
+namespace mi_ep {
+namespace {
+
+constexpr uint32_t kFlagAggregate = 1;
+constexpr uint32_t kFlagPrefix = 2;
+constexpr uint32_t kGenMask = 0x3fffffffu;
+
+__device__ __forceinline__ uint64_t pack_status(uint32_t flag, uint32_t gen, uint32_t value) {
+  return (static_cast<uint64_t>(flag) << 62) | (static_cast<uint64_t>(gen & kGenMask) << 32) |
+         static_cast<uint64_t>(value);
+}
+__device__ __forceinline__ void publish(uint64_t* p, uint64_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t peek(const uint64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Lanes of the wave that hold the same valid expert as this lane (including it).
+// Executed by all lanes; the result is meaningful only where `valid`.
+__device__ __forceinline__ uint64_t match_expert(bool valid, int e, int expert_bits) {
+  uint64_t mask = __ballot(valid);
+  for (int b = 0; b < expert_bits; ++b) {
+    const bool bit = ((e >> b) & 1) != 0;
+    const uint64_t with_bit = __ballot(valid && bit);
+    mask &= bit ? with_bit : ~with_bit;
+  }
+  return mask;
+}
+
+__device__ __forceinline__ void store_token_flags(uint8_t* is_token_in_rank, int token,
+                                                  int num_ranks, uint64_t flags) {
+  uint8_t* dst = is_token_in_rank + static_cast<size_t>(token) * num_ranks;
+  if (num_ranks == 8 && (reinterpret_cast<uintptr_t>(is_token_in_rank) & 7u) == 0) {
+    *reinterpret_cast<uint64_t*>(dst) = flags;
+  } else if (num_ranks == 4 && (reinterpret_cast<uintptr_t>(is_token_in_rank) & 3u) == 0) {
+    *reinterpret_cast<uint32_t*>(dst) = static_cast<uint32_t>(flags);
+  } else {
+    for (int r = 0; r < num_ranks; ++r) dst[r] = static_cast<uint8_t>((flags >> (8 * r)) & 1u);
+  }
+}
+
+__global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const LayoutArgs a) {
+  extern __shared__ int smem[];
+  const int E = a.num_experts, R = a.num_ranks, K = a.num_topk, T = a.num_tokens;
+  const int cols = E + R;
+  int* hist = smem;                         // [kLayoutWaves][E] wave-private counters
+  int* col_total = hist + kLayoutWaves * E; // [cols] this tile's total per column
+  int* col_excl = col_total + cols;         // [cols] sum over earlier tiles
+  int* rank_cnt = col_excl + cols;          // [kMaxRanks]
+  int* wave_sums = rank_cnt + kMaxRanks;    // [kLayoutWaves]
+  int* misc = wave_sums + kLayoutWaves;     // [4] tile, generation
+  uint64_t* tok_flags = reinterpret_cast<uint64_t*>(misc + 4);  // [kTileTokens], byte r = rank r
+
+  const int tid = static_cast<int>(threadIdx.x);
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  uint64_t* status = reinterpret_cast<uint64_t*>(a.ws + 1);
+
+  if (tid == 0) {
+    misc[1] = static_cast<int>(
+        __hip_atomic_load(&a.ws->generation, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kGenMask);
+    misc[0] = static_cast<int>(
+        __hip_atomic_fetch_add(&a.ws->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  }
+  for (int i = tid; i < kLayoutWaves * E; i += kLayoutThreads) hist[i] = 0;
+  if (tid < kMaxRanks) rank_cnt[tid] = 0;
+  tok_flags[tid] = 0;
+  __syncthreads();
+
+  const int tile = misc[0];
+  const uint32_t gen = static_cast<uint32_t>(misc[1]);
+  if (tile >= a.num_tiles) return;  // stale ticket: never with an initialised workspace
+  const int t0 = tile * kTileTokens;
+  const int flat0 = t0 * K;
+  const int flat_end = T * K;
+  int* my_hist = hist + wave * E;
+
+  // ---- routes of this wave, 64 per chunk, in (token, slot) order ----------
+  int my_e[kMaxTopk];
+  int my_pos[kMaxTopk];
+#pragma unroll
+  for (int c = 0; c < kMaxTopk; ++c) {
+    my_e[c] = -1;
+    my_pos[c] = 0;
+    if (c < K) {
+      const int local = (wave * K + c) * kWave + lane;
+      const int g = flat0 + local;
+      const int64_t e64 = (g < flat_end) ? a.topk_idx[g] : -1;
+      const bool valid = e64 >= 0 && e64 < static_cast<int64_t>(E);
+      const int e = valid ? static_cast<int>(e64) : 0;
+      const uint64_t same = match_expert(valid, e, a.expert_bits);
+      int old = 0, below = 0;
+      if (valid) {
+        below = __popcll(same & lanes_below(lane));
+        old = my_hist[e];
+        my_e[c] = e;
+        my_pos[c] = old + below;
+        reinterpret_cast<uint8_t*>(tok_flags + local / K)[e / a.experts_per_rank] = 1;
+      }
+      __builtin_amdgcn_wave_barrier();
+      if (valid && below == 0) my_hist[e] = old + __popcll(same);
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+  __syncthreads();
+
+  // ---- flags out, de-duplicated rank hits ------------------------------------
+  {
+    const int t = t0 + tid;
+    const uint64_t f = tok_flags[tid];
+    if (t < T) store_token_flags(a.is_token_in_rank, t, R, f);
+    for (int r = 0; r < R; ++r) {
+      const uint64_t hit = __ballot(((f >> (8 * r)) & 1u) != 0);
+      if (lane == 0 && hit != 0) atomicAdd(&rank_cnt[r], __popcll(hit));
+    }
+  }
+  __syncthreads();
+
+  // ---- per column: tile total, wave bases, decoupled look-back ----------------
+  for (int col = tid; col < cols; col += kLayoutThreads) {
+    int total = 0;
+    if (col < E) {
+#pragma unroll
+      for (int w = 0; w < kLayoutWaves; ++w) {
+        const int v = hist[w * E + col];
+        hist[w * E + col] = total;  // becomes the wave's base inside the tile
+        total += v;
+      }
+    } else {
+      total = rank_cnt[col - E];
+    }
+    uint64_t* mine = status + static_cast<size_t>(tile) * cols + col;
+    int excl = 0;
+    if (tile == 0) {
+      publish(mine, pack_status(kFlagPrefix, gen, static_cast<uint32_t>(total)));
+    } else {
+      publish(mine, pack_status(kFlagAggregate, gen, static_cast<uint32_t>(total)));
+      for (int j = tile - 1; j >= 0; --j) {
+        const uint64_t* theirs = status + static_cast<size_t>(j) * cols + col;
+        uint64_t s = peek(theirs);
+        uint32_t spins = 0;
+        while ((static_cast<uint32_t>(s >> 32) & kGenMask) != gen || (s >> 62) == 0) {
+          if (++spins > a.spin_limit) {
+            __hip_atomic_store(&a.ws->timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s = pack_status(kFlagPrefix, gen, 0u);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
+          s = peek(theirs);
+        }
+        excl += static_cast<int>(static_cast<uint32_t>(s));
+        if ((s >> 62) == kFlagPrefix) break;
+      }
+      publish(mine, pack_status(kFlagPrefix, gen, static_cast<uint32_t>(excl + total)));
+    }
+    col_excl[col] = excl;
+    col_total[col] = total;
+  }
+  __syncthreads();
+
+  // ---- position of every route inside its expert segment --------------------
+  if (a.slot_rel != nullptr) {
+#pragma unroll
+    for (int c = 0; c < kMaxTopk; ++c) {
+      if (c < K) {
+        const int g = flat0 + (wave * K + c) * kWave + lane;
+        if (g < flat_end) {
+          const int e = my_e[c];
+          a.slot_rel[g] = (e >= 0) ? col_excl[e] + my_hist[e] + my_pos[c] : -1;
+        }
+      }
+    }
+  }
+
+  // ---- per-channel inclusive prefix: the tile holding a channel's end writes it
+  if (a.channel_prefix_matrix != nullptr) {
+    const int C = a.num_channels;
+    const int per_channel = (T + C - 1) / C;
+    for (int idx = tid; idx < C * R; idx += kLayoutThreads) {
+      const int c = idx / R, r = idx - c * R;
+      const long long s64 = static_cast<long long>(per_channel) * c;
+      const int start = s64 < T ? static_cast<int>(s64) : T;
+      const int end = (T - start < per_channel) ? T : start + per_channel;
+      if (end > t0 && end <= t0 + kTileTokens) {
+        int cnt = 0;
+        for (int tl = 0; tl < end - t0; ++tl) cnt += static_cast<int>((tok_flags[tl] >> (8 * r)) & 1u);
+        a.channel_prefix_matrix[r * C + c] = col_excl[E + r] + cnt;
+      }
+    }
+  }
+
+  // ---- the last tile owns the grand totals ----------------------------------
+  if (tile == a.num_tiles - 1) {
+    for (int col = tid; col < cols; col += kLayoutThreads) {
+      const int cnt = col_excl[col] + col_total[col];
+      if (col < E)
+        a.num_tokens_per_expert[col] = cnt;
+      else
+        a.num_tokens_per_rank[col - E] = cnt;
+    }
+    if (a.expert_offsets != nullptr) {
+      // Block-wide exclusive scan of the aligned counts; each thread owns a run
+      // of consecutive experts so that the scan order is the expert order.
+      const int per_thread = (E + kLayoutThreads - 1) / kLayoutThreads;
+      const int first = tid * per_thread;
+      const int align = a.expert_alignment;
+      int local = 0;
+      for (int i = 0; i < per_thread; ++i) {
+        const int e = first + i;
+        if (e < E) {
+          const int cnt = col_excl[e] + col_total[e];
+          local += (cnt + align - 1) / align * align;
+        }
+      }
+      int incl = local;
+#pragma unroll
+      for (int d = 1; d < kWave; d <<= 1) {
+        const int up = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += up;
+      }
+      if (lane == kWave - 1) wave_sums[wave] = incl;
+      __syncthreads();
+      int base = incl - local;
+      int grand = 0;
+#pragma unroll
+      for (int w = 0; w < kLayoutWaves; ++w) {
+        if (w < wave) base += wave_sums[w];
+        grand += wave_sums[w];
+      }
+      int* offs = hist;  // wave bases are no longer needed by this tile
+      __syncthreads();
+      for (int i = 0; i < per_thread; ++i) {
+        const int e = first + i;
+        if (e < E) {
+          offs[e] = base;
+          a.expert_offsets[e] = base;
+          const int cnt = col_excl[e] + col_total[e];
+          base += (cnt + align - 1) / align * align;
+        }
+      }
+      if (tid == 0) {
+        offs[E] = grand;
+        a.expert_offsets[E] = grand;
+      }
+      __syncthreads();
+      if (a.psum_rank_rows != nullptr && tid < R)
+        a.psum_rank_rows[tid] = offs[(tid + 1) * a.experts_per_rank];
+    }
+  }
+
+  // ---- hand the workspace back ready for the next launch --------------------
+  __syncthreads();
+  if (tid == 0) {
+    const uint32_t finished =
+        __hip_atomic_fetch_add(&a.ws->done, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    if (finished == static_cast<uint32_t>(a.num_tiles) - 1u) {
+      __hip_atomic_store(&a.ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&a.ws->done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&a.ws->generation, (gen + 1u) & kGenMask, __ATOMIC_RELEASE,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// Counts and flags only, accumulated with global atomics into zeroed outputs.
+__global__ __launch_bounds__(kLayoutThreads) void ep_layout_counts_kernel(
+    const int64_t* __restrict__ topk_idx, int* num_tokens_per_rank, int* num_tokens_per_expert,
+    uint8_t* is_token_in_rank, int T, int K, int R, int E, int experts_per_rank, int expert_bits,
+    int num_tiles) {
+  extern __shared__ int smem[];
+  int* hist = smem;                // [E]
+  int* rank_cnt = hist + E;        // [kMaxRanks]
+  uint64_t* tok_flags = reinterpret_cast<uint64_t*>(rank_cnt + kMaxRanks + (E & 1));  // [kTileTokens]
+  const int tid = static_cast<int>(threadIdx.x);
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+
+  for (int i = tid; i < E; i += kLayoutThreads) hist[i] = 0;
+  if (tid < kMaxRanks) rank_cnt[tid] = 0;
+  const int flat_end = T * K;
+  for (int tile = static_cast<int>(blockIdx.x); tile < num_tiles; tile += static_cast<int>(gridDim.x)) {
+    tok_flags[tid] = 0;
+    __syncthreads();
+    const int t0 = tile * kTileTokens;
+    const int flat0 = t0 * K;
+    for (int c = 0; c < K; ++c) {
+      const int local = (wave * K + c) * kWave + lane;
+      const int g = flat0 + local;
+      const int64_t e64 = (g < flat_end) ? topk_idx[g] : -1;
+      const bool valid = e64 >= 0 && e64 < static_cast<int64_t>(E);
+      const int e = valid ? static_cast<int>(e64) : 0;
+      const uint64_t same = match_expert(valid, e, expert_bits);
+      if (valid) {
+        if ((same & lanes_below(lane)) == 0) atomicAdd(&hist[e], __popcll(same));
+        reinterpret_cast<uint8_t*>(tok_flags + local / K)[e / experts_per_rank] = 1;
+      }
+    }
+    __syncthreads();
+    const int t = t0 + tid;
+    const uint64_t f = tok_flags[tid];
+    if (t < T) store_token_flags(is_token_in_rank, t, R, f);
+    for (int r = 0; r < R; ++r) {
+      const uint64_t hit = __ballot(((f >> (8 * r)) & 1u) != 0);
+      if (lane == 0 && hit != 0) atomicAdd(&rank_cnt[r], __popcll(hit));
+    }
+    __syncthreads();
+  }
+  __syncthreads();
+  for (int i = tid; i < E; i += kLayoutThreads)
+    if (hist[i] != 0) atomicAdd(&num_tokens_per_expert[i], hist[i]);
+  if (tid < R && rank_cnt[tid] != 0) atomicAdd(&num_tokens_per_rank[tid], rank_cnt[tid]);
+}
+
+__global__ void ep_fill_u32_kernel(uint32_t* dst, size_t count, uint32_t value) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += stride)
+    dst[i] = value;
+}
+
+__global__ void ep_zero_counts_kernel(int* a, int na, int* b, int nb) {
+  const int i = static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
+  if (i < na) a[i] = 0;
+  if (i < nb) b[i] = 0;
+}
+
+}  // namespace
+
+hipError_t launch_fill_u32(uint32_t* dst, size_t count, uint32_t value, hipStream_t stream) {
+  if (count == 0) return hipSuccess;
+  const int threads = 256;
+  size_t blocks = (count + threads - 1) / threads;
+  if (blocks > 2048) blocks = 2048;
+  hipLaunchKernelGGL(ep_fill_u32_kernel, dim3(static_cast<unsigned>(blocks)), dim3(threads), 0, stream,
+                     dst, count, value);
+  return hipGetLastError();
+}
+
+hipError_t launch_layout_fused(const LayoutArgs& a, hipStream_t stream) {
+  const int cols = a.num_experts + a.num_ranks;
+  const size_t lds = sizeof(int) * (static_cast<size_t>(kLayoutWaves) * a.num_experts + 2 * cols +
+                                    kMaxRanks + kLayoutWaves + 4) +
+                     sizeof(uint64_t) * kTileTokens;
+  hipLaunchKernelGGL(ep_layout_fused_kernel, dim3(a.num_tiles), dim3(kLayoutThreads), lds, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_layout_counts(const int64_t* topk_idx, int* num_tokens_per_rank,
+                                int* num_tokens_per_expert, uint8_t* is_token_in_rank,
+                                int num_tokens, int num_topk, int num_ranks, int num_experts,
+                                hipStream_t stream) {
+  const int n = num_experts > num_ranks ? num_experts : num_ranks;
+  hipLaunchKernelGGL(ep_zero_counts_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
+                     num_tokens_per_expert, num_experts, num_tokens_per_rank, num_ranks);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess || num_tokens == 0) return err;
+  const int num_tiles = (num_tokens + kTileTokens - 1) / kTileTokens;
+  int expert_bits = 1;
+  while ((1 << expert_bits) < num_experts) ++expert_bits;
+  const int grid = num_tiles < 1024 ? num_tiles : 1024;
+  const size_t lds = sizeof(int) * (num_experts + kMaxRanks + (num_experts & 1)) +
+                     sizeof(uint64_t) * kTileTokens;
+  hipLaunchKernelGGL(ep_layout_counts_kernel, dim3(grid), dim3(kLayoutThreads), lds, stream, topk_idx,
+                     num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, num_tokens, num_topk,
+                     num_ranks, num_experts, num_experts / num_ranks, expert_bits, num_tiles);
+  return hipGetLastError();
+}
+
+}  // namespace mi_ep

@@ -1,0 +1,261 @@
+"""Host-side operator surface over the C ABI (include/mi_ep.h).
+
+Mirrors the DeepEP-style operators the reference drives
+(datasets/example080_deepep_jit_dispatch_payload/nv/build_and_run.py:710-732,
+datasets/example082_deepep_jit_combine/nv/build_and_run.py:751-765) for one GPU whose HBM is
+split into `num_ranks` partitions:
+
+    get_dispatch_layout(topk_idx, num_experts, num_ranks)
+        -> (num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank)
+    dispatch(x, scales, topk_idx, topk_weights, ...)
+        -> (recv_x, recv_scales, recv_src_map, handle)
+    combine(y, slot_map | handle, topk_weights) -> combined_x
+
+torch is used for device memory and streams only; all arithmetic runs in the HIP kernels of
+libmi_ep.so.  Nothing here falls back to torch ops or to the CPU.
+"""
+from dataclasses import dataclass
+from typing import Optional, Tuple, Union
+
+import torch
+
+from . import _lib
+
+MAX_RANKS = 8
+MAX_TOPK = 8
+MAX_EXPERTS = 1024
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _check_routing(topk_idx: torch.Tensor, num_experts: int, num_ranks: int) -> Tuple[int, int]:
+    _require(topk_idx.is_cuda, "topk_idx must live on the GPU")
+    _require(topk_idx.dtype == torch.int64 and topk_idx.dim() == 2 and topk_idx.is_contiguous(),
+             "topk_idx must be a contiguous int64 [num_tokens, num_topk] tensor")
+    # Same wording as the reference's constructor checks (example042 .cu:96-107).
+    _require(0 < num_ranks <= MAX_RANKS, f"num_ranks must be in [1, {MAX_RANKS}]")
+    _require(0 < topk_idx.shape[1] <= MAX_TOPK, f"num_topk must be in [1, {MAX_TOPK}]")
+    _require(num_experts > 0 and num_experts % num_ranks == 0,
+             "num_experts must be divisible by num_ranks")
+    _require(num_experts <= MAX_EXPERTS, f"num_experts must be at most {MAX_EXPERTS}")
+    return topk_idx.shape[0], topk_idx.shape[1]
+
+
+def get_dispatch_layout(topk_idx: torch.Tensor, num_experts: int, num_ranks: int):
+    """Counts and flags only; the reference's DeepepDispatchLayout::compute (example042 .cu:110-132)."""
+    T, K = _check_routing(topk_idx, num_experts, num_ranks)
+    dev = topk_idx.device
+    per_rank = torch.empty(num_ranks, dtype=torch.int32, device=dev)
+    per_expert = torch.empty(num_experts, dtype=torch.int32, device=dev)
+    in_rank = torch.empty((T, num_ranks), dtype=torch.bool, device=dev)
+    lib = _lib.load()
+    _lib.check(lib.mi_ep_get_dispatch_layout(_ptr(topk_idx), _ptr(per_rank), None, _ptr(per_expert),
+                                             _ptr(in_rank), T, K, num_ranks, num_experts, _stream()),
+               "mi_ep_get_dispatch_layout")
+    return per_rank, per_expert, in_rank
+
+
+@dataclass
+class DispatchHandle:
+    """State carried from dispatch to combine (the reference's `handle`, example082 bar.py:744-755)."""
+    num_tokens: int
+    num_topk: int
+    num_experts: int
+    num_ranks: int
+    expert_alignment: int
+    num_tokens_per_rank: torch.Tensor      # int32[R]
+    num_tokens_per_expert: torch.Tensor    # int32[E]
+    is_token_in_rank: torch.Tensor         # bool[T, R]
+    expert_offsets: torch.Tensor           # int32[E + 1], exclusive over aligned counts
+    psum_rank_rows: torch.Tensor           # int32[R], inclusive rows per partition
+    channel_prefix_matrix: Optional[torch.Tensor]  # int32[R, C]
+    slot_rel: torch.Tensor                 # int32[T, K]
+    slot_map: Optional[torch.Tensor] = None        # int32[T, K]
+    recv_src_map: Optional[torch.Tensor] = None    # int32[capacity]
+    recv_topk_idx: Optional[torch.Tensor] = None   # int64[capacity]
+    recv_topk_weights: Optional[torch.Tensor] = None  # float32[capacity]
+
+    def num_recv_rows(self) -> int:
+        """Padded row total; synchronises the stream."""
+        return int(self.expert_offsets[-1].item())
+
+
+class Buffer:
+    """Workspace owner, the one-GPU analogue of the reference's ElasticBuffer
+    (example080 bar.py:683-693).  Calls on one Buffer must not overlap in time."""
+
+    def __init__(self, num_max_tokens: int, num_topk: int, num_experts: int, num_ranks: int,
+                 device: Union[str, torch.device] = "cuda"):
+        _require(0 < num_ranks <= MAX_RANKS, f"num_ranks must be in [1, {MAX_RANKS}]")
+        _require(0 < num_topk <= MAX_TOPK, f"num_topk must be in [1, {MAX_TOPK}]")
+        _require(num_experts > 0 and num_experts % num_ranks == 0,
+                 "num_experts must be divisible by num_ranks")
+        _require(num_experts <= MAX_EXPERTS, f"num_experts must be at most {MAX_EXPERTS}")
+        self.num_max_tokens = num_max_tokens
+        self.num_topk = num_topk
+        self.num_experts = num_experts
+        self.num_ranks = num_ranks
+        self.device = torch.device(device)
+        lib = _lib.load()
+        nbytes = lib.mi_ep_workspace_bytes(max(num_max_tokens, 1), num_topk, num_experts, num_ranks)
+        _require(nbytes > 0, "unsupported shape")
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        with torch.cuda.device(self.device):
+            _lib.check(lib.mi_ep_workspace_init(_ptr(self.workspace), nbytes, _stream()),
+                       "mi_ep_workspace_init")
+
+    def status(self) -> None:
+        """Raises if a device-side bounded wait ever expired on this workspace."""
+        lib = _lib.load()
+        with torch.cuda.device(self.device):
+            _lib.check(lib.mi_ep_workspace_status(_ptr(self.workspace), _stream()),
+                       "mi_ep_workspace_status")
+
+    def dispatch_layout(self, topk_idx: torch.Tensor, expert_alignment: int = 1,
+                        num_channels: int = 0) -> DispatchHandle:
+        """Fused single-pass layout: counts, flags, offsets, per-route segment positions."""
+        T, K = _check_routing(topk_idx, self.num_experts, self.num_ranks)
+        _require(K == self.num_topk, "num_topk differs from the buffer's")
+        _require(T <= self.num_max_tokens, "more tokens than the buffer was sized for")
+        _require(expert_alignment >= 1, "expert_alignment must be positive")
+        E, R, dev = self.num_experts, self.num_ranks, topk_idx.device
+        h = DispatchHandle(
+            num_tokens=T, num_topk=K, num_experts=E, num_ranks=R, expert_alignment=expert_alignment,
+            num_tokens_per_rank=torch.empty(R, dtype=torch.int32, device=dev),
+            num_tokens_per_expert=torch.empty(E, dtype=torch.int32, device=dev),
+            is_token_in_rank=torch.empty((T, R), dtype=torch.bool, device=dev),
+            expert_offsets=torch.empty(E + 1, dtype=torch.int32, device=dev),
+            psum_rank_rows=torch.empty(R, dtype=torch.int32, device=dev),
+            channel_prefix_matrix=(torch.empty((R, num_channels), dtype=torch.int32, device=dev)
+                                   if num_channels > 0 else None),
+            slot_rel=torch.empty((T, K), dtype=torch.int32, device=dev),
+        )
+        lib = _lib.load()
+        _lib.check(lib.mi_ep_dispatch_layout(
+            _ptr(topk_idx), T, K, R, E, expert_alignment, num_channels,
+            _ptr(h.num_tokens_per_rank), _ptr(h.num_tokens_per_expert), _ptr(h.is_token_in_rank),
+            _ptr(h.expert_offsets), _ptr(h.psum_rank_rows), _ptr(h.channel_prefix_matrix),
+            _ptr(h.slot_rel), _ptr(self.workspace), self.workspace.numel(), _stream()),
+            "mi_ep_dispatch_layout")
+        return h
+
+    def dispatch(self, x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Tensor,
+                 topk_weights: Optional[torch.Tensor], expert_alignment: int = 1,
+                 num_channels: int = 0, handle: Optional[DispatchHandle] = None,
+                 capacity_rows: Optional[int] = None):
+        """Layout (unless `handle` is given) + permute into the expert-contiguous buffer.
+
+        Returns (recv_x, recv_scales, recv_src_map, handle).  Buffers hold `capacity_rows` rows
+        (default: the worst case T*K + E*(alignment-1), so no host sync is needed); rows at and
+        beyond handle.num_recv_rows() are unspecified.
+        """
+        if handle is None:
+            handle = self.dispatch_layout(topk_idx, expert_alignment, num_channels)
+        T, K, E = handle.num_tokens, handle.num_topk, handle.num_experts
+        _require(x.is_cuda and x.dim() == 2 and x.is_contiguous() and x.shape[0] == T,
+                 "x must be a contiguous [num_tokens, hidden] GPU tensor")
+        row_bytes = x.shape[1] * x.element_size()
+        _require(row_bytes % 16 == 0, "row size must be a multiple of 16 bytes")
+        num_scales = 0
+        if scales is not None:
+            _require(scales.dtype == torch.float32 and scales.dim() == 2 and scales.is_contiguous()
+                     and scales.shape[0] == T, "scales must be contiguous float32 [num_tokens, S]")
+            num_scales = scales.shape[1]
+        if topk_weights is not None:
+            _require(topk_weights.dtype == torch.float32 and topk_weights.is_contiguous()
+                     and tuple(topk_weights.shape) == (T, K),
+                     "topk_weights must be contiguous float32 [num_tokens, num_topk]")
+        if capacity_rows is None:
+            capacity_rows = T * K + E * (handle.expert_alignment - 1)
+        dev = x.device
+        recv_x = torch.empty((capacity_rows, x.shape[1]), dtype=x.dtype, device=dev)
+        recv_scales = (torch.empty((capacity_rows, num_scales), dtype=torch.float32, device=dev)
+                       if scales is not None else None)
+        handle.recv_src_map = torch.empty(capacity_rows, dtype=torch.int32, device=dev)
+        handle.recv_topk_idx = torch.empty(capacity_rows, dtype=torch.int64, device=dev)
+        handle.recv_topk_weights = torch.empty(capacity_rows, dtype=torch.float32, device=dev)
+        handle.slot_map = torch.empty((T, K), dtype=torch.int32, device=dev)
+        lib = _lib.load()
+        _lib.check(lib.mi_ep_dispatch(
+            _ptr(x), _ptr(scales), _ptr(topk_idx), _ptr(topk_weights), _ptr(handle.expert_offsets),
+            _ptr(handle.slot_rel), _ptr(handle.num_tokens_per_expert), T, K, E,
+            handle.expert_alignment, row_bytes, num_scales, _ptr(recv_x), _ptr(recv_scales),
+            _ptr(handle.recv_src_map), _ptr(handle.recv_topk_idx), _ptr(handle.recv_topk_weights),
+            _ptr(handle.slot_map), capacity_rows, _stream()), "mi_ep_dispatch")
+        return recv_x, recv_scales, handle.recv_src_map, handle
+
+
+def combine(y: torch.Tensor, slot_map: Union[torch.Tensor, DispatchHandle],
+            topk_weights: Optional[torch.Tensor] = None,
+            bias: Union[None, torch.Tensor, Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]] = None,
+            recv_topk_weights: Optional[torch.Tensor] = None):
+    """combined_x[t] = bf16(sum_k w[t,k] * y[slot_map[t,k]] (+ biases)), fp32 accumulation.
+
+    topk_weights=None gives the reference's plain ordered sum.  When `recv_topk_weights` (the
+    per-row weights that travelled with dispatch) is given, also returns them gathered back to
+    [num_tokens, num_topk], as the reference's combined_topk_weights.
+    """
+    if isinstance(slot_map, DispatchHandle):
+        _require(slot_map.slot_map is not None, "handle has not been through dispatch")
+        slot_map = slot_map.slot_map
+    _require(y.is_cuda and y.dtype == torch.bfloat16 and y.dim() == 2 and y.is_contiguous(),
+             "y must be a contiguous bf16 [rows, hidden] GPU tensor")
+    _require(slot_map.dtype == torch.int32 and slot_map.dim() == 2 and slot_map.is_contiguous(),
+             "slot_map must be contiguous int32 [num_tokens, num_topk]")
+    T, K = slot_map.shape
+    _require(0 < K <= MAX_TOPK, f"num_topk must be in [1, {MAX_TOPK}]")
+    H = y.shape[1]
+    _require(H % 8 == 0, "hidden must be a multiple of 8")
+    if topk_weights is not None:
+        _require(topk_weights.dtype == torch.float32 and topk_weights.is_contiguous()
+                 and tuple(topk_weights.shape) == (T, K),
+                 "topk_weights must be contiguous float32 [num_tokens, num_topk]")
+    bias_0 = bias_1 = None
+    if isinstance(bias, torch.Tensor):
+        bias_0 = bias
+    elif bias is not None:
+        bias_0, bias_1 = bias
+    for b in (bias_0, bias_1):
+        if b is not None:
+            _require(b.dtype == torch.bfloat16 and b.is_contiguous() and tuple(b.shape) == (T, H),
+                     "bias must be contiguous bf16 [num_tokens, hidden]")
+    dev = y.device
+    out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    out_w = (torch.empty((T, K), dtype=torch.float32, device=dev)
+             if recv_topk_weights is not None else None)
+    lib = _lib.load()
+    _lib.check(lib.mi_ep_combine(_ptr(y), _ptr(slot_map), _ptr(topk_weights), _ptr(bias_0),
+                                 _ptr(bias_1), _ptr(recv_topk_weights), T, K, H, _ptr(out),
+                                 _ptr(out_w), _stream()), "mi_ep_combine")
+    if out_w is not None:
+        return out, out_w
+    return out
+
+
+def dispatch(x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Tensor,
+             topk_weights: Optional[torch.Tensor], num_experts: int, num_ranks: int,
+             expert_alignment: int = 1, num_channels: int = 0):
+    """One-shot form: allocates a Buffer for this call's shape.  Prefer Buffer.dispatch in loops."""
+    T, K = _check_routing(topk_idx, num_experts, num_ranks)
+    buf = Buffer(T, K, num_experts, num_ranks, device=topk_idx.device)
+    return buf.dispatch(x, scales, topk_idx, topk_weights, expert_alignment, num_channels)
+
+
+def copy_yardstick(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """16-byte streaming copy of src into dst (same byte size), the measured-bandwidth yardstick."""
+    nbytes = src.numel() * src.element_size()
+    _require(dst.numel() * dst.element_size() == nbytes and nbytes % 16 == 0, "size mismatch")
+    lib = _lib.load()
+    _lib.check(lib.mi_ep_copy_yardstick(_ptr(dst), _ptr(src), nbytes, _stream()),
+               "mi_ep_copy_yardstick")

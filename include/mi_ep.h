@@ -1,0 +1,150 @@
+/*
+ * mi_ep.h -- C ABI of the MI355X (gfx950) expert-parallel dispatch core.
+ *
+ * One GPU; the reference's "ranks" are partitions of this GPU's HBM.  Every
+ * pointer is a device pointer unless stated otherwise, every call enqueues on
+ * `stream` (a hipStream_t passed as void*, NULL = the null stream) and returns
+ * without synchronising.  The caller owns every buffer.  Return value: 0 on
+ * success, a negative MI_EP_E* code for bad arguments, a positive hipError_t
+ * when the HIP runtime reports one.  Nothing here exits the process.
+ *
+ * Reference files are cited relative to the reference tree's datasets/ folder.
+ */
+#ifndef MI_EP_H_
+#define MI_EP_H_
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI_EP_ABI_VERSION 1
+
+#define MI_EP_OK 0
+#define MI_EP_EINVAL (-22)    /* argument out of range or NULL where required */
+#define MI_EP_ENOSPC (-28)    /* workspace too small */
+#define MI_EP_ETIMEDOUT (-110) /* device-side bounded wait expired (mi_ep_workspace_status) */
+
+/* Limits.  Ranks and top-k follow the reference's constructor checks
+ * (example042_deepep_dispatch_layout/nv/empty_deepep_dispatch_layout.cu:43,46,96-107). */
+#define MI_EP_MAX_RANKS 8
+#define MI_EP_MAX_TOPK 8
+#define MI_EP_MAX_EXPERTS 1024
+
+int mi_ep_abi_version(void);
+const char* mi_ep_strerror(int code);
+
+/*
+ * Dispatch layout, exact kernel-level signature of
+ * example042_deepep_dispatch_layout/nv/empty_deepep_dispatch_layout.cu:48-58
+ * (deepep_get_dispatch_layout_kernel) plus the stream of
+ * DeepepDispatchLayout::compute (:110-132).
+ *   topk_idx                  int64[num_tokens, num_topk]; < 0 = masked slot
+ *   num_tokens_per_rank       int32[num_ranks]   one per (token, rank) pair
+ *   num_tokens_per_rdma_rank  accepted and ignored (always NULL in the reference)
+ *   num_tokens_per_expert     int32[num_experts] every valid slot counts
+ *   is_token_in_rank          bool[num_tokens, num_ranks]
+ * Outputs are overwritten, not accumulated into (the reference benchmark never
+ * re-zeroes them, :313-329).  Needs no workspace.
+ */
+int mi_ep_get_dispatch_layout(const int64_t* topk_idx, int* num_tokens_per_rank,
+                              int* num_tokens_per_rdma_rank, int* num_tokens_per_expert,
+                              bool* is_token_in_rank, int num_tokens, int num_topk, int num_ranks,
+                              int num_experts, void* stream);
+
+/*
+ * Workspace of the fused layout kernel below.  It must be initialised once
+ * (mi_ep_workspace_init) before its first use; every later call leaves it ready
+ * for the next.  Calls that share one workspace must not overlap in time.
+ */
+size_t mi_ep_workspace_bytes(int num_tokens, int num_topk, int num_experts, int num_ranks);
+int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+/* Synchronises `stream`, then reports MI_EP_ETIMEDOUT if any launch on this
+ * workspace gave up a bounded device-side wait since the last init. */
+int mi_ep_workspace_status(const void* workspace, void* stream);
+
+/*
+ * Fused single-pass layout: everything the reference spreads over
+ *   example042 (counts + flags, empty_deepep_dispatch_layout.cu:48-86),
+ *   example047 (per-channel inclusive prefix, empty_deepep_intranode_notify_dispatch.cu:132-143),
+ *   example078 (deterministic slots, empty_deepep_jit_dispatch_deterministic_prologue.cu:27-43),
+ *   example080 notify role (histogram, aligned exclusive expert psum, inclusive rank
+ *   psum, empty_deepep_jit_dispatch_payload.cu:78-107,197-239).
+ * Outputs (any of the last four may be NULL):
+ *   num_tokens_per_rank / num_tokens_per_expert / is_token_in_rank   as above
+ *   expert_offsets      int32[num_experts + 1]; off[0] = 0,
+ *                       off[e+1] = off[e] + round_up(count[e], expert_alignment)
+ *   psum_rank_rows      int32[num_ranks]; inclusive rows of partitions 0..r
+ *   channel_prefix_matrix int32[num_ranks, num_channels]; tokens flagged for rank r in
+ *                       token tiles 0..c (tile bounds as get_channel_task_range, :73-79)
+ *   slot_rel            int32[num_tokens, num_topk]; position of route (t,k) inside its
+ *                       expert segment in (token, slot) order, -1 for non-routes
+ */
+int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
+                          int num_experts, int expert_alignment, int num_channels,
+                          int* num_tokens_per_rank, int* num_tokens_per_expert,
+                          bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
+                          int* channel_prefix_matrix, int* slot_rel, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/*
+ * Dispatch (permute): the payload role of dispatch_impl
+ * (example080_deepep_jit_dispatch_payload/nv/empty_deepep_jit_dispatch_payload.cu:31-44,241-256)
+ * fused with dispatch_copy_epilogue_impl in expand mode
+ * (example081_deepep_jit_dispatch_copy_epilogue/nv/empty_deepep_jit_dispatch_copy_epilogue.cu:22-60).
+ * Row slot_map[t,k] = expert_offsets[e] + slot_rel[t,k] of every output receives
+ * token t's input; segment e is rows [off[e], off[e+1]).
+ *   x            [num_tokens, row_bytes] opaque bytes (bf16 or fp8); row_bytes % 16 == 0,
+ *                x and recv_x 16-byte aligned
+ *   x_scales     float[num_tokens, num_scales] or NULL (num_scales = 0)
+ *   topk_weights float[num_tokens, num_topk] or NULL
+ *   recv_x       [capacity_rows, row_bytes]
+ *   recv_scales  float[capacity_rows, num_scales] or NULL
+ *   recv_src_map int32[capacity_rows]: source token of each row; -1 for pad rows
+ *   recv_topk_idx     int64[capacity_rows] or NULL: expert owning the row; -1 pad
+ *   recv_topk_weights float[capacity_rows] or NULL: gate weight of the row's route; 0 pad
+ *   slot_map     int32[num_tokens, num_topk]: absolute row of each route, -1 non-routes
+ * Rows >= capacity_rows are never written.  With expert_alignment > 1 pad rows are
+ * zero-filled; num_tokens_per_expert (from the layout call) locates them and may be
+ * NULL when expert_alignment == 1.
+ */
+int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
+                   const float* topk_weights, const int* expert_offsets, const int* slot_rel,
+                   const int* num_tokens_per_expert, int num_tokens, int num_topk,
+                   int num_experts, int expert_alignment, int row_bytes, int num_scales,
+                   void* recv_x, float* recv_scales, int* recv_src_map, int64_t* recv_topk_idx,
+                   float* recv_topk_weights, int* slot_map, int capacity_rows, void* stream);
+
+/*
+ * Combine: combine_impl + combine_reduce_epilogue_impl
+ * (example082_deepep_jit_combine/nv/empty_deepep_jit_combine.cu:28-67,
+ *  example083_deepep_jit_combine_reduce_epilogue/nv/empty_deepep_jit_combine_reduce_epilogue.cu:23-53).
+ *   combined_x[t,h] = bf16( sum_k w[t,k] * y[slot_map[t,k], h] + bias_0[t,h] + bias_1[t,h] )
+ * accumulated in fp32, slots ascending, one fused multiply-add per row, one
+ * rounding to bf16 at the end.  topk_weights == NULL gives the reference's plain
+ * ordered sum.  hidden % 8 == 0; y, biases and combined_x 16-byte aligned.
+ *   y            bf16[*, hidden] expert outputs in dispatch row order
+ *   bias_0/1     bf16[num_tokens, hidden] or NULL
+ *   recv_topk_weights / combined_topk_weights   both NULL, or float[rows] in and
+ *                float[num_tokens, num_topk] out: the weights that travelled with the
+ *                rows, gathered back per route (0 for non-routes)
+ */
+int mi_ep_combine(const void* y, const int* slot_map, const float* topk_weights,
+                  const void* bias_0, const void* bias_1, const float* recv_topk_weights,
+                  int num_tokens, int num_topk, int hidden, void* combined_x,
+                  float* combined_topk_weights, void* stream);
+
+/*
+ * 16-byte streaming copy used as the measured HBM ceiling next to the nominal
+ * peak; same access width as example077_GPU_vectorized_copy_widths (16-byte loads).
+ * bytes % 16 == 0.
+ */
+int mi_ep_copy_yardstick(void* dst, const void* src, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_EP_H_ */

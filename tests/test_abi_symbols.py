@@ -1,0 +1,71 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/mi_ep.h declares."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mi_ep.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi_ep_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_surface():
+    names = declared_functions()
+    for required in ("mi_ep_get_dispatch_layout", "mi_ep_dispatch_layout", "mi_ep_dispatch",
+                     "mi_ep_combine", "mi_ep_workspace_bytes", "mi_ep_workspace_init"):
+        assert required in names
+
+
+def test_library_exports_every_declared_symbol():
+    from commbench_amd import _lib
+    assert os.path.exists(_lib.LIB_PATH), "build with `python -m commbench_amd.build`"
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} declared in mi_ep.h but not exported"
+    assert sorted(_lib.SIGNATURES) == declared_functions()
+
+
+def test_host_only_entry_points():
+    """Calls that touch no device: version, error strings, workspace sizing, argument checks."""
+    from commbench_amd import _lib
+    lib = _lib.load()
+    assert lib.mi_ep_abi_version() == 1
+    assert _lib.strerror(0) == "ok"
+    assert _lib.strerror(-22) == "invalid argument"
+    assert _lib.strerror(-28) == "workspace too small"
+    # 256-byte header + ceil(T/256) tiles x (E + R) 8-byte status words
+    assert lib.mi_ep_workspace_bytes(8192, 8, 256, 8) == 256 + 32 * 264 * 8
+    assert lib.mi_ep_workspace_bytes(1, 1, 1, 1) == 256 + 1 * 2 * 8
+    assert lib.mi_ep_workspace_bytes(8192, 8, 256, 9) == 0       # more than 8 ranks
+    assert lib.mi_ep_workspace_bytes(8192, 9, 256, 8) == 0       # more than 8 slots
+    assert lib.mi_ep_workspace_bytes(8192, 8, 250, 8) == 0       # experts not divisible by ranks
+    # Argument errors are reported before any launch.
+    assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 2, 9, 18, None) == -22
+    assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 9, 2, 8, None) == -22
+    assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 2, 3, 8, None) == -22
+    assert lib.mi_ep_dispatch_layout(None, 4, 2, 2, 8, 0, 0, None, None, None, None, None, None,
+                                     None, None, 0, None) == -22     # alignment 0
+    assert lib.mi_ep_combine(None, None, None, None, None, None, 4, 2, 12, None, None, None) == -22
+    assert lib.mi_ep_dispatch(None, None, None, None, None, None, None, 4, 2, 8, 1, 24, 0,
+                              None, None, None, None, None, None, 0, None) == -22   # 24 % 16 != 0
+
+
+def test_python_surface_rejects_bad_arguments_like_the_reference():
+    """Same conditions and wording as the reference's constructor checks (example042 .cu:96-107)."""
+    import torch
+    from commbench_amd import ops
+    topk = torch.zeros((4, 2), dtype=torch.int64)
+    with pytest.raises(ValueError, match="GPU"):
+        ops.get_dispatch_layout(topk, 8, 2)
+    with pytest.raises(ValueError, match=r"num_ranks must be in \[1, 8\]"):
+        ops.Buffer(16, 2, 18, 9, device="cpu")
+    with pytest.raises(ValueError, match=r"num_topk must be in \[1, 8\]"):
+        ops.Buffer(16, 9, 16, 8, device="cpu")
+    with pytest.raises(ValueError, match="divisible"):
+        ops.Buffer(16, 2, 10, 4, device="cpu")

@@ -1,0 +1,220 @@
+"""GPU parity of permute and combine (through the C ABI) against the CPU checker.
+
+Bars: maps, side data and permuted payload bit-exact; combine within 2 bf16 ulp of the
+fp32-accumulated host result (the kernel uses the same fused multiply-add chain, so the tests
+also report whether it was bit-exact).
+"""
+import numpy as np
+import pytest
+import torch
+
+from commbench_amd import ops
+from commbench_amd import workloads as wl
+
+from . import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+
+COMBINE_ULP_TOLERANCE = 2
+
+
+def dispatch_and_check(oracle, cfg_or_shape, topk_np, w_np, x_cpu, scales_cpu, align=1):
+    """Runs layout + permute on the GPU, compares everything with the checker, returns both."""
+    T, K = topk_np.shape
+    E, R = cfg_or_shape
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    topk = torch.from_numpy(topk_np).to(gu.DEV)
+    w = torch.from_numpy(w_np).to(gu.DEV) if w_np is not None else None
+    x = x_cpu.to(gu.DEV)
+    scales = scales_cpu.to(gu.DEV) if scales_cpu is not None else None
+    recv_x, recv_scales, recv_src_map, h = buf.dispatch(x, scales, topk, w, expert_alignment=align)
+    torch.cuda.synchronize()
+    buf.status()
+    ref = oracle.full_path(topk_np, w_np, gu.as_bytes(x_cpu),
+                           None if scales_cpu is None else scales_cpu.numpy(), E, R, align)
+    rows = int(ref["expert_offsets"][-1])
+    assert h.num_recv_rows() == rows
+    np.testing.assert_array_equal(h.slot_map.cpu().numpy(), ref["slot_map"])
+    np.testing.assert_array_equal(recv_src_map.cpu().numpy()[:rows], ref["recv_src_map"])
+    np.testing.assert_array_equal(h.recv_topk_idx.cpu().numpy()[:rows], ref["recv_topk_idx"])
+    np.testing.assert_array_equal(gu.as_bytes(recv_x)[:rows], ref["recv_x"])
+    if scales_cpu is not None:
+        np.testing.assert_array_equal(recv_scales.cpu().numpy()[:rows].view(np.uint32),
+                                      ref["recv_scales"].view(np.uint32))
+    if w_np is not None:
+        np.testing.assert_array_equal(h.recv_topk_weights.cpu().numpy()[:rows].view(np.uint32),
+                                      ref["recv_topk_weights"].view(np.uint32))
+    return recv_x, h, ref
+
+
+def combine_and_check(oracle, y_gpu, slot_map_gpu, w_np, ref_slot_map, biases=(None, None)):
+    w = torch.from_numpy(w_np).to(gu.DEV) if w_np is not None else None
+    b_gpu = tuple(None if b is None else b.to(gu.DEV) for b in biases)
+    out = ops.combine(y_gpu, slot_map_gpu, w, bias=b_gpu)
+    torch.cuda.synchronize()
+    want = oracle.combine(gu.bf16_bits(y_gpu), ref_slot_map, w_np,
+                          *[None if b is None else gu.bf16_bits(b) for b in biases], num_threads=8)
+    got = gu.bf16_bits(out)
+    dist = gu.bf16_ulp_distance(got, want)
+    assert dist.max() <= COMBINE_ULP_TOLERANCE, f"max distance {dist.max()} bf16 ulp"
+    return got, want, int(dist.max())
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c5"])
+def test_bf16_configs_dispatch_then_combine(oracle, name):
+    cfg = wl.CONFIGS[name]
+    print(f"config {name}", flush=True)
+    topk_np, w_np = wl.make_routing(cfg)
+    x_cpu, _ = wl.make_payload(cfg)
+    recv_x, h, ref = dispatch_and_check(oracle, (cfg.num_experts, cfg.num_ranks), topk_np, w_np, x_cpu, None)
+    rows = int(ref["expert_offsets"][-1])
+    if cfg.expert_scale_denom > 0:
+        # expert e multiplies its rows by 1 + e / denom (fp32 multiply, one rounding to bf16)
+        e_of_row = h.recv_topk_idx[:rows].to(torch.float32)
+        scale = 1.0 + e_of_row / cfg.expert_scale_denom
+        y = (recv_x[:rows].to(torch.float32) * scale[:, None]).to(torch.bfloat16)
+        want_y = oracle.scale_rows_by_expert(ref["recv_x"].view(np.uint16), ref["expert_offsets"],
+                                             cfg.expert_scale_denom, num_threads=8)
+        np.testing.assert_array_equal(gu.bf16_bits(y), want_y)
+    else:
+        y = recv_x[:rows]                         # identity experts
+    got, want, worst = combine_and_check(oracle, y.contiguous(), h.slot_map, w_np, ref["slot_map"])
+    print(f"{name}: combine max distance {worst} ulp, bit-exact={bool((got == want).all())}", flush=True)
+    if cfg.expert_scale_denom == 0 and cfg.mask_prob == 0:
+        # identity experts + gates summing to 1: the round trip returns x to within 2 ulp
+        xb = gu.bf16_bits(x_cpu)
+        assert gu.bf16_ulp_distance(got, xb).max() <= 2
+
+
+def test_fp8_config_with_scales(oracle):
+    cfg = wl.CONFIGS["c4"]
+    topk_np, w_np = wl.make_routing(cfg)
+    q_cpu, scales_cpu = wl.make_payload(cfg)
+    assert q_cpu.dtype == torch.float8_e4m3fn and scales_cpu.shape == (cfg.num_tokens, 56)
+    _, h, ref = dispatch_and_check(oracle, (cfg.num_experts, cfg.num_ranks), topk_np, w_np, q_cpu, scales_cpu)
+    rows = int(ref["expert_offsets"][-1])
+    y = wl.make_expert_outputs(cfg, rows).to(gu.DEV)          # combine consumes fresh bf16 outputs
+    combine_and_check(oracle, y, h.slot_map, w_np, ref["slot_map"])
+
+
+@pytest.mark.parametrize("align", [2, 128])
+def test_alignment_pads_are_zero_rows(oracle, align):
+    rng = np.random.default_rng(align)
+    T, K, E, R, H = 777, 8, 64, 8, 512
+    topk_np = wl.zipf_distinct_topk(rng, T, E, K, 1.2)
+    topk_np[rng.random((T, K)) < 0.05] = -1
+    w_np = wl.softmax_gates(rng, T, K)
+    x_cpu = wl.bf16_normal(rng, T, H)
+    recv_x, h, ref = dispatch_and_check(oracle, (E, R), topk_np, w_np, x_cpu, None, align=align)
+    off = ref["expert_offsets"]
+    assert (off % align == 0).all()
+    pads = ref["recv_src_map"] < 0
+    assert pads.any() and not gu.as_bytes(recv_x)[:off[-1]][pads].any()
+
+
+@pytest.mark.parametrize("shape", [
+    # T, K, E, R, row_bytes, num_scales
+    (1, 1, 1, 1, 16, 0), (5, 3, 6, 2, 48, 1), (300, 8, 32, 4, 1024, 8), (300, 8, 32, 4, 1040, 0),
+    (129, 2, 8, 8, 2064, 70), (64, 7, 1024, 8, 14336, 0)], ids=lambda s: "x".join(map(str, s)))
+def test_permute_ragged_shapes(oracle, shape):
+    T, K, E, R, row_bytes, S = shape
+    print(f"shape {shape}", flush=True)
+    rng = np.random.default_rng(sum(shape))
+    topk_np = rng.integers(-1, E, size=(T, K)).astype(np.int64)
+    w_np = rng.standard_normal((T, K)).astype(np.float32)
+    x_cpu = torch.from_numpy(rng.integers(0, 256, size=(T, row_bytes), dtype=np.uint8))
+    scales_cpu = torch.from_numpy(rng.standard_normal((T, S)).astype(np.float32)) if S else None
+    dispatch_and_check(oracle, (E, R), topk_np, w_np, x_cpu, scales_cpu, align=1)
+
+
+def test_capacity_limits_writes(oracle):
+    """Rows at or beyond capacity_rows are dropped: never written, slot_map = -1."""
+    rng = np.random.default_rng(3)
+    T, K, E, R, H = 200, 4, 16, 4, 64
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    x = wl.bf16_normal(rng, T, H).to(gu.DEV)
+    topk = torch.from_numpy(topk_np).to(gu.DEV)
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    cap = 500
+    recv_x, _, src_map, h = buf.dispatch(x, None, topk, None, capacity_rows=cap)
+    torch.cuda.synchronize()
+    ref = oracle.full_path(topk_np, None, gu.as_bytes(x), None, E, R)
+    want_slots = np.where(ref["slot_map"] < cap, ref["slot_map"], -1)
+    np.testing.assert_array_equal(h.slot_map.cpu().numpy(), want_slots)
+    np.testing.assert_array_equal(gu.as_bytes(recv_x), ref["recv_x"][:cap])
+    np.testing.assert_array_equal(src_map.cpu().numpy(), ref["recv_src_map"][:cap])
+
+
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_combine_every_topk_with_biases(oracle, K):
+    rng = np.random.default_rng(K)
+    T, E, R, H = 333, 32, 4, 1096            # 137 vectors per row: ragged last batch
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    topk_np[rng.random((T, K)) < 0.15] = -1
+    w_np = wl.softmax_gates(rng, T, K)
+    _, per_expert, _ = oracle.layout(topk_np, R, E)
+    off, _ = oracle.expert_offsets(per_expert, R, 1)
+    _, slot_map, _, _ = oracle.slot_maps(topk_np, E, off)
+    y = wl.bf16_normal(rng, int(off[-1]) + 3, H).to(gu.DEV)
+    b0, b1 = wl.bf16_normal(rng, T, H), wl.bf16_normal(rng, T, H)
+    sm = torch.from_numpy(slot_map).to(gu.DEV)
+    for weights, biases in ((w_np, (None, None)), (None, (None, None)), (w_np, (b0, None)), (w_np, (b0, b1))):
+        got, want, worst = combine_and_check(oracle, y, sm, weights, slot_map, biases)
+        assert worst == 0, "same fma chain on both sides: expected bit-exact"
+
+
+def test_combine_integer_payload_is_exact(oracle):
+    rng = np.random.default_rng(21)
+    T, K, E, R, H = 500, 8, 64, 8, 256
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    _, per_expert, _ = oracle.layout(topk_np, R, E)
+    off, _ = oracle.expert_offsets(per_expert, R, 1)
+    _, slot_map, _, _ = oracle.slot_maps(topk_np, E, off)
+    y_int = rng.integers(-15, 16, size=(int(off[-1]), H))
+    y = torch.from_numpy(y_int.astype(np.float32)).to(torch.bfloat16).to(gu.DEV)
+    out = ops.combine(y, torch.from_numpy(slot_map).to(gu.DEV), None)
+    want = y_int[slot_map.reshape(-1)].reshape(T, K, H).sum(axis=1)
+    np.testing.assert_array_equal(out.to(torch.float32).cpu().numpy(), want)
+
+
+def test_combine_returns_travelled_weights(oracle):
+    """The reference's harness expects combined_topk_weights == topk_weights
+    (example082 build_and_run.py:764-765); masked slots come back as 0."""
+    rng = np.random.default_rng(8)
+    T, K, E, R, H = 257, 8, 64, 8, 128
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    topk_np[rng.random((T, K)) < 0.1] = -1
+    w_np = wl.softmax_gates(rng, T, K)
+    x_cpu = wl.bf16_normal(rng, T, H)
+    recv_x, h, ref = dispatch_and_check(oracle, (E, R), topk_np, w_np, x_cpu, None)
+    rows = int(ref["expert_offsets"][-1])
+    out, out_w = ops.combine(recv_x[:rows].contiguous(), h, None, recv_topk_weights=h.recv_topk_weights)
+    want_w = np.where(topk_np >= 0, w_np, 0).astype(np.float32)
+    np.testing.assert_array_equal(out_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    np.testing.assert_array_equal(out_w.cpu().numpy(), oracle.gather_weights(ref["recv_topk_weights"], ref["slot_map"]))
+
+
+def test_full_size_properties_without_the_checker():
+    """Target shape (8192 x 7168 bf16, 256 experts, top-8): properties that need no CPU pass.
+    K = 8 distinct experts, gates = 1/8 exactly: permute then combine returns x bit-for-bit
+    (eight equal fma steps of x/8 are exact in fp32), every row is written exactly once."""
+    cfg = wl.CONFIGS["target"]
+    T, K, E, R, H = cfg.num_tokens, cfg.num_topk, cfg.num_experts, cfg.num_ranks, cfg.hidden
+    topk_np, _ = wl.make_routing(cfg)
+    gen = torch.Generator(device=gu.DEV).manual_seed(1)
+    x = torch.randn((T, H), device=gu.DEV, generator=gen, dtype=torch.float32).to(torch.bfloat16)
+    topk = torch.from_numpy(topk_np).to(gu.DEV)
+    w = torch.full((T, K), 0.125, dtype=torch.float32, device=gu.DEV)
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    recv_x, _, src_map, h = buf.dispatch(x, None, topk, w)
+    torch.cuda.synchronize()
+    assert h.num_recv_rows() == T * K
+    sm = h.slot_map.reshape(-1).to(torch.int64)
+    assert torch.equal(torch.sort(sm).values, torch.arange(T * K, device=gu.DEV))   # a permutation
+    assert torch.equal(src_map.to(torch.int64)[sm], torch.arange(T * K, device=gu.DEV) // K)
+    assert torch.equal(recv_x.view(torch.int16)[sm[::K]], x.view(torch.int16))     # slot 0 rows
+    seg = h.recv_topk_idx[:T * K]
+    assert torch.equal(seg, torch.sort(seg).values)                                 # expert-contiguous
+    assert torch.equal(torch.bincount(seg, minlength=E).to(torch.int32), h.num_tokens_per_expert)
+    out = ops.combine(recv_x, h, w)
+    assert torch.equal(out.view(torch.int16), x.view(torch.int16))

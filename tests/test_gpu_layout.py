@@ -1,0 +1,132 @@
+"""GPU parity of the layout kernels (through the C ABI) against the CPU checker: bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from commbench_amd import ops
+from commbench_amd import workloads as wl
+
+from . import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+
+
+# ---- the reference's own correctness cases, on its own operator surface ---------------------
+
+@pytest.mark.parametrize("case", wl.REFERENCE_LAYOUT_CASES, ids=lambda c: "-".join(map(str, c)))
+def test_get_dispatch_layout_reference_cases(oracle, case):
+    T, K, R, E, pattern = case
+    print(f"case {case}", flush=True)
+    topk_np = wl.reference_pattern_topk(T, K, R, E, pattern)
+    topk = torch.from_numpy(topk_np).to(gu.DEV)
+    per_rank, per_expert, flags = ops.get_dispatch_layout(topk, E, R)
+    torch.cuda.synchronize()
+    w_rank, w_expert, w_flags = oracle.layout(topk_np, R, E)
+    np.testing.assert_array_equal(per_rank.cpu().numpy(), w_rank)
+    np.testing.assert_array_equal(per_expert.cpu().numpy(), w_expert)
+    np.testing.assert_array_equal(flags.cpu().numpy().view(np.uint8), w_flags)
+
+
+def test_get_dispatch_layout_overwrites_its_outputs(oracle):
+    """The reference's benchmark relaunches without re-zeroing (example042 .cu:313-329)."""
+    from commbench_amd import _lib
+    T, K, R, E = 1000, 4, 4, 64
+    topk_np = wl.uniform_distinct_topk(np.random.default_rng(0), T, E, K)
+    topk = torch.from_numpy(topk_np).to(gu.DEV)
+    per_rank = torch.full((R,), 12345, dtype=torch.int32, device=gu.DEV)
+    per_expert = torch.full((E,), -777, dtype=torch.int32, device=gu.DEV)
+    flags = gu.garbage_like(torch.empty((T, R), dtype=torch.bool, device=gu.DEV)).view(torch.uint8)
+    lib = _lib.load()
+    for _ in range(3):
+        _lib.check(lib.mi_ep_get_dispatch_layout(topk.data_ptr(), per_rank.data_ptr(), None,
+                                                 per_expert.data_ptr(), flags.data_ptr(), T, K, R, E,
+                                                 torch.cuda.current_stream().cuda_stream), "layout")
+    torch.cuda.synchronize()
+    w_rank, w_expert, w_flags = oracle.layout(topk_np, R, E)
+    np.testing.assert_array_equal(per_rank.cpu().numpy(), w_rank)
+    np.testing.assert_array_equal(per_expert.cpu().numpy(), w_expert)
+    np.testing.assert_array_equal(flags.cpu().numpy().reshape(T, R), w_flags)
+
+
+# ---- fused single-pass layout --------------------------------------------------------------
+
+@pytest.mark.parametrize("case", wl.REFERENCE_LAYOUT_CASES, ids=lambda c: "-".join(map(str, c)))
+def test_fused_layout_reference_cases(oracle, case):
+    T, K, R, E, pattern = case
+    print(f"case {case}", flush=True)
+    topk_np = wl.reference_pattern_topk(T, K, R, E, pattern)
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    _, h = gu.run_fused_layout(buf, topk_np, expert_alignment=1, num_channels=2 * R)
+    gu.check_layout_against_oracle(oracle, h, topk_np, R, E, 1, 2 * R)
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+def test_fused_layout_configs(oracle, name):
+    cfg = wl.CONFIGS[name]
+    print(f"config {name}", flush=True)
+    topk_np, _ = wl.make_routing(cfg)
+    buf = ops.Buffer(cfg.num_tokens, cfg.num_topk, cfg.num_experts, cfg.num_ranks, device=gu.DEV)
+    for align in (1, 128):
+        _, h = gu.run_fused_layout(buf, topk_np, expert_alignment=align, num_channels=16)
+        gu.check_layout_against_oracle(oracle, h, topk_np, cfg.num_ranks, cfg.num_experts, align, 16)
+
+
+@pytest.mark.parametrize("shape", [
+    (1, 1, 1, 1), (1, 8, 8, 8), (7, 2, 2, 4), (255, 3, 1, 5), (256, 8, 8, 1024), (257, 5, 4, 12),
+    (513, 7, 2, 6), (3000, 6, 8, 1024), (65536, 2, 8, 32)], ids=lambda s: "x".join(map(str, s)))
+def test_fused_layout_ragged_shapes(oracle, shape):
+    T, K, R, E = shape
+    print(f"shape {shape}", flush=True)
+    rng = np.random.default_rng(T * 31 + K)
+    topk_np = rng.integers(-1, E, size=(T, K)).astype(np.int64)     # masks and duplicates
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    _, h = gu.run_fused_layout(buf, topk_np, expert_alignment=3, num_channels=5)
+    gu.check_layout_against_oracle(oracle, h, topk_np, R, E, 3, 5)
+
+
+def test_fused_layout_out_of_range_and_all_masked(oracle):
+    T, K, R, E = 700, 4, 4, 16
+    rng = np.random.default_rng(5)
+    topk_np = rng.integers(-3, E + 3, size=(T, K)).astype(np.int64)
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    _, h = gu.run_fused_layout(buf, topk_np)
+    gu.check_layout_against_oracle(oracle, h, topk_np, R, E)
+    masked = np.full((T, K), -1, dtype=np.int64)
+    _, h = gu.run_fused_layout(buf, masked)
+    ref = gu.check_layout_against_oracle(oracle, h, masked, R, E)
+    assert ref["off"][-1] == 0
+
+
+def test_fused_layout_zero_tokens(oracle):
+    buf = ops.Buffer(16, 2, 8, 2, device=gu.DEV)
+    empty = np.zeros((0, 2), dtype=np.int64)
+    _, h = gu.run_fused_layout(buf, empty, expert_alignment=4, num_channels=4)
+    assert not h.num_tokens_per_expert.cpu().numpy().any()
+    assert not h.expert_offsets.cpu().numpy().any()
+    assert not h.channel_prefix_matrix.cpu().numpy().any()
+
+
+def test_workspace_is_reusable_across_shapes_and_many_calls(oracle):
+    """One workspace, alternating token counts: status words of earlier launches must never be
+    mistaken for this launch's."""
+    K, R, E = 8, 8, 64
+    buf = ops.Buffer(5000, K, E, R, device=gu.DEV)
+    rng = np.random.default_rng(17)
+    for i, T in enumerate([5000, 300, 4097, 1, 5000, 2048, 300, 5000] * 3):
+        topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+        _, h = gu.run_fused_layout(buf, topk_np)
+        gu.check_layout_against_oracle(oracle, h, topk_np, R, E)
+
+
+@pytest.mark.parametrize("T", [7, 4096, 4097])
+@pytest.mark.parametrize("R", [2, 4, 8])
+def test_channel_prefix_reference_notify_cases(oracle, T, R):
+    """The reference's notify inputs (example047 .cu:599-610): two destinations per token."""
+    C = wl.reference_notify_channels(R)
+    flags = wl.reference_notify_flags(T, R, 0)
+    t = np.arange(T)
+    topk_np = np.stack([t % R, (t + 1) % R], axis=1).astype(np.int64)    # one expert per rank
+    buf = ops.Buffer(T, 2, R, R, device=gu.DEV)
+    _, h = gu.run_fused_layout(buf, topk_np, num_channels=C)
+    np.testing.assert_array_equal(h.is_token_in_rank.cpu().numpy().view(np.uint8), flags)
+    np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy(), oracle.channel_prefix(flags, C))
