@@ -28,6 +28,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="target")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
 
@@ -181,10 +182,42 @@ def main():
         wk.step()
     torch.cuda.synchronize()
 
-    # Timed region: exactly `steps` steps; HIP events on the launch stream bracket each kernel.
-    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    # Timed region: exactly `steps` steps, back to back on one stream.
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    for _ in range(args.steps):
+        wk.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # The same steps replayed as one HIP graph of the three kernels (no host launch gaps).
+    graph_ms_per_step = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            wk.stream = side.cuda_stream
+            wk.step()
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                wk.stream = torch.cuda.current_stream().cuda_stream
+                wk.step()
+        wk.stream = torch.cuda.current_stream().cuda_stream
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # Per-kernel durations: the same steps again with HIP events on the launch stream
+    # bracketing every kernel (kept out of the region above, where they would add gaps).
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
     for ev in marks:
         ev[0].record()
         wk.layout()
@@ -194,8 +227,6 @@ def main():
         wk.combine()
         ev[3].record()
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
 
     names = ["ep_layout_fused_kernel", "ep_permute_kernel", "ep_combine_kernel"]
     kernel_us = {n: sum(ev[i].elapsed_time(ev[i + 1]) for ev in marks) * 1e3 / args.steps
@@ -248,6 +279,7 @@ def main():
         },
         "hbm_gbps_whole_step": wk.bytes["total"] / (ms_per_step * 1e-3) / 1e9,
         "hbm_frac_whole_step": wk.bytes["total"] / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+        "graph_replay_ms_per_step": graph_ms_per_step,
         "algorithmic_bytes": wk.bytes,
         "kernel_us": kernel_us,
         "kernel_gbps": {n: kernel_bytes[n] / (kernel_us[n] * 1e-6) / 1e9 for n in names},

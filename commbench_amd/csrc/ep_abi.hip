@@ -80,7 +80,7 @@ int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream) 
 int mi_ep_workspace_status(const void* workspace, void* stream) {
   if (workspace == nullptr) return MI_EP_EINVAL;
   LayoutWorkspace header;
-  hipError_t e = hipMemcpyAsync(&header, workspace, sizeof(uint32_t) * 4, hipMemcpyDeviceToHost,
+  hipError_t e = hipMemcpyAsync(&header, workspace, sizeof(uint64_t) * 2, hipMemcpyDeviceToHost,
                                 as_stream(stream));
   if (e != hipSuccess) return static_cast<int>(e);
   e = hipStreamSynchronize(as_stream(stream));
@@ -145,6 +145,8 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
   a.num_tiles = num_tiles_for(num_tokens);
   a.expert_bits = 1;
   while ((1 << a.expert_bits) < num_experts) ++a.expert_bits;
+  a.inv_topk = ((1u << 19) + num_topk - 1) / num_topk;
+  a.inv_experts_per_rank = ((1u << 22) + a.experts_per_rank - 1) / a.experts_per_rank;
   a.spin_limit = kSpinLimit;
   return status_of(launch_layout_fused(a, s));
 }

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kCombineThreads) void ep_combine_kernel(const Combi
       vec16 out;
 #pragma unroll
       for (int i = 0; i < 4; ++i) out[i] = pack_bf16(acc[u][2 * i], acc[u][2 * i + 1]);
-      __builtin_nontemporal_store(out, a.combined_x + o);
+      a.combined_x[o] = out;
     }
   }
 }

@@ -16,16 +16,19 @@ constexpr int kMaxTopk = 8;
 constexpr int kMaxExperts = 1024;
 
 // ---- layout ---------------------------------------------------------------
-constexpr int kLayoutThreads = 256;
+constexpr int kLayoutThreads = 1024;
 constexpr int kLayoutWaves = kLayoutThreads / kWave;
-constexpr int kTileTokens = 256;  // one token per thread of the tile's workgroup
+constexpr int kTileTokens = 256;
+// A tile's 256 * K routes are 4 * K chunks of 64, shared out over the 16 waves.
+constexpr int kChunksPerWave = ((kTileTokens / kWave) * kMaxTopk + kLayoutWaves - 1) / kLayoutWaves;
 
 // Header of the fused layout kernel's workspace; the look-back status words follow.
+// `turn` packs {generation:32 | ticket:32}: one fetch-add hands a tile both its
+// index and the launch's generation; the tile that draws the last ticket stores
+// {generation + 1, 0}, which is safe because every ticket of the launch is out.
 struct alignas(256) LayoutWorkspace {
-  uint32_t ticket;      // next tile to hand out
-  uint32_t done;        // tiles finished in the running launch
-  uint32_t generation;  // bumped by the last tile of every launch
-  uint32_t timed_out;   // sticky: a bounded wait expired
+  uint64_t turn;
+  uint32_t timed_out;  // sticky: a bounded wait expired
 };
 
 struct LayoutArgs {
@@ -47,6 +50,8 @@ struct LayoutArgs {
   int num_channels;
   int num_tiles;
   int expert_bits;  // ceil(log2(num_experts)), at least 1
+  uint32_t inv_topk;              // ceil(2^19 / num_topk): n / num_topk == (n * inv) >> 19 for n < 2048
+  uint32_t inv_experts_per_rank;  // ceil(2^22 / experts_per_rank): exact for e < 1024
   uint32_t spin_limit;
 };
 

@@ -10,11 +10,13 @@
 // (example047 .cu:132-143).
 //
 // Shape of the computation (wave64):
-//   * a tile is 256 tokens = 256*K routes, owned by one 256-thread workgroup;
+//   * a tile is 256 tokens = 256*K routes, owned by one 1024-thread workgroup;
 //     tiles are handed out by an atomic ticket so that every tile's predecessors
 //     have already started, which makes the look-back below deadlock-free
-//     whatever the residency of the grid;
-//   * each wave walks its 64*K routes in 64-route chunks in (token, slot) order;
+//     whatever the residency of the grid; the same fetch-add returns the
+//     launch's generation, and the last ticket holder resets the word;
+//   * the workgroup is 16 waves; each walks its share of the tile's 4*K chunks
+//     of 64 routes in (token, slot) order;
 //     lanes holding the same expert find each other with log2(E) ballots, the
 //     lowest such lane bumps the wave's private LDS counter once, and every lane
 //     derives its rank among equals with a popcount -- no LDS atomics, so routing
@@ -36,6 +38,8 @@ namespace {
 constexpr uint32_t kFlagAggregate = 1;
 constexpr uint32_t kFlagPrefix = 2;
 constexpr uint32_t kGenMask = 0x3fffffffu;
+constexpr int kLookbackWindow = 32;
+constexpr int kCountsThreads = 256;  // the counts-only kernel: one token per thread, 4 waves
 
 __device__ __forceinline__ uint64_t pack_status(uint32_t flag, uint32_t gen, uint32_t value) {
   return (static_cast<uint64_t>(flag) << 62) | (static_cast<uint64_t>(gen & kGenMask) << 32) |
@@ -76,13 +80,14 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   extern __shared__ int smem[];
   const int E = a.num_experts, R = a.num_ranks, K = a.num_topk, T = a.num_tokens;
   const int cols = E + R;
-  int* hist = smem;                         // [kLayoutWaves][E] wave-private counters
-  int* col_total = hist + kLayoutWaves * E; // [cols] this tile's total per column
+  int* col_total = smem;                    // [cols] this tile's total per column
   int* col_excl = col_total + cols;         // [cols] sum over earlier tiles
   int* rank_cnt = col_excl + cols;          // [kMaxRanks]
   int* wave_sums = rank_cnt + kMaxRanks;    // [kLayoutWaves]
   int* misc = wave_sums + kLayoutWaves;     // [4] tile, generation
-  uint64_t* tok_flags = reinterpret_cast<uint64_t*>(misc + 4);  // [kTileTokens], byte r = rank r
+  int* offs = misc + 4;                     // [E + 2] offsets staged by the last tile
+  uint64_t* tok_flags = reinterpret_cast<uint64_t*>(offs + E + 2 + (E & 1));  // [kTileTokens], byte r = rank r
+  uint16_t* hist = reinterpret_cast<uint16_t*>(tok_flags + kTileTokens);  // [kLayoutWaves][E] wave-private
 
   const int tid = static_cast<int>(threadIdx.x);
   const int lane = tid & (kWave - 1);
@@ -90,14 +95,23 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   uint64_t* status = reinterpret_cast<uint64_t*>(a.ws + 1);
 
   if (tid == 0) {
-    misc[1] = static_cast<int>(
-        __hip_atomic_load(&a.ws->generation, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kGenMask);
-    misc[0] = static_cast<int>(
-        __hip_atomic_fetch_add(&a.ws->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    const uint64_t turn =
+        __hip_atomic_fetch_add(&a.ws->turn, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t ticket = static_cast<uint32_t>(turn);
+    const uint32_t generation = static_cast<uint32_t>(turn >> 32) & kGenMask;
+    misc[0] = static_cast<int>(ticket);
+    misc[1] = static_cast<int>(generation);
+    // Last ticket of the launch: hand the workspace to the next launch.
+    if (ticket == static_cast<uint32_t>(a.num_tiles) - 1u)
+      __hip_atomic_store(&a.ws->turn, static_cast<uint64_t>((generation + 1u) & kGenMask) << 32,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  for (int i = tid; i < kLayoutWaves * E; i += kLayoutThreads) hist[i] = 0;
+  {
+    uint32_t* hist_words = reinterpret_cast<uint32_t*>(hist);
+    for (int i = tid; i < (kLayoutWaves * E + 1) / 2; i += kLayoutThreads) hist_words[i] = 0;
+  }
   if (tid < kMaxRanks) rank_cnt[tid] = 0;
-  tok_flags[tid] = 0;
+  if (tid < kTileTokens) tok_flags[tid] = 0;
   __syncthreads();
 
   const int tile = misc[0];
@@ -106,19 +120,32 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   const int t0 = tile * kTileTokens;
   const int flat0 = t0 * K;
   const int flat_end = T * K;
-  int* my_hist = hist + wave * E;
+  uint16_t* my_hist = hist + wave * E;
 
-  // ---- routes of this wave, 64 per chunk, in (token, slot) order ----------
-  int my_e[kMaxTopk];
-  int my_pos[kMaxTopk];
+  // ---- routes: the tile's 256*K routes are 4*K chunks of 64 in (token, slot)
+  // order; wave w owns chunks [w * per_wave, (w + 1) * per_wave).
+  const int num_chunks = (kTileTokens / kWave) * K;
+  const int per_wave = (num_chunks + kLayoutWaves - 1) / kLayoutWaves;  // <= kChunksPerWave
+  int64_t raw[kChunksPerWave];
 #pragma unroll
-  for (int c = 0; c < kMaxTopk; ++c) {
+  for (int c = 0; c < kChunksPerWave; ++c) {
+    raw[c] = -1;
+    const int chunk = wave * per_wave + c;
+    if (c < per_wave && chunk < num_chunks) {
+      const int g = flat0 + chunk * kWave + lane;
+      if (g < flat_end) raw[c] = a.topk_idx[g];
+    }
+  }
+  int my_e[kChunksPerWave];
+  int my_pos[kChunksPerWave];
+#pragma unroll
+  for (int c = 0; c < kChunksPerWave; ++c) {
     my_e[c] = -1;
     my_pos[c] = 0;
-    if (c < K) {
-      const int local = (wave * K + c) * kWave + lane;
-      const int g = flat0 + local;
-      const int64_t e64 = (g < flat_end) ? a.topk_idx[g] : -1;
+    const int chunk = wave * per_wave + c;
+    if (c < per_wave && chunk < num_chunks) {  // wave-uniform
+      const int local = chunk * kWave + lane;  // < 256 * K <= 2048
+      const int64_t e64 = raw[c];
       const bool valid = e64 >= 0 && e64 < static_cast<int64_t>(E);
       const int e = valid ? static_cast<int>(e64) : 0;
       const uint64_t same = match_expert(valid, e, a.expert_bits);
@@ -128,17 +155,20 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
         old = my_hist[e];
         my_e[c] = e;
         my_pos[c] = old + below;
-        reinterpret_cast<uint8_t*>(tok_flags + local / K)[e / a.experts_per_rank] = 1;
+        // local / K and e / experts_per_rank by multiply-shift (exact on these ranges)
+        const int token_local = static_cast<int>((static_cast<uint32_t>(local) * a.inv_topk) >> 19);
+        const int rank = static_cast<int>((static_cast<uint32_t>(e) * a.inv_experts_per_rank) >> 22);
+        reinterpret_cast<uint8_t*>(tok_flags + token_local)[rank] = 1;
       }
       __builtin_amdgcn_wave_barrier();
-      if (valid && below == 0) my_hist[e] = old + __popcll(same);
+      if (valid && below == 0) my_hist[e] = static_cast<uint16_t>(old + __popcll(same));
       __builtin_amdgcn_wave_barrier();
     }
   }
   __syncthreads();
 
-  // ---- flags out, de-duplicated rank hits ------------------------------------
-  {
+  // ---- flags out, de-duplicated rank hits (one token per thread) ---------------
+  if (tid < kTileTokens) {
     const int t = t0 + tid;
     const uint64_t f = tok_flags[tid];
     if (t < T) store_token_flags(a.is_token_in_rank, t, R, f);
@@ -156,7 +186,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
 #pragma unroll
       for (int w = 0; w < kLayoutWaves; ++w) {
         const int v = hist[w * E + col];
-        hist[w * E + col] = total;  // becomes the wave's base inside the tile
+        hist[w * E + col] = static_cast<uint16_t>(total);  // becomes the wave's base inside the tile
         total += v;
       }
     } else {
@@ -168,21 +198,42 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
       publish(mine, pack_status(kFlagPrefix, gen, static_cast<uint32_t>(total)));
     } else {
       publish(mine, pack_status(kFlagAggregate, gen, static_cast<uint32_t>(total)));
-      for (int j = tile - 1; j >= 0; --j) {
-        const uint64_t* theirs = status + static_cast<size_t>(j) * cols + col;
-        uint64_t s = peek(theirs);
-        uint32_t spins = 0;
-        while ((static_cast<uint32_t>(s >> 32) & kGenMask) != gen || (s >> 62) == 0) {
+      // Fold predecessors in, nearest first, a window of independent loads at a
+      // time so that one memory round trip covers kLookbackWindow tiles.  "Tile -1"
+      // is an empty prefix, which ends the walk at the front of the grid.
+      int next = tile - 1;
+      uint32_t spins = 0;
+      bool found_prefix = false;
+      while (!found_prefix) {
+        uint64_t s[kLookbackWindow];
+#pragma unroll
+        for (int i = 0; i < kLookbackWindow; ++i) {
+          const int j = next - i;
+          s[i] = (j >= 0) ? peek(status + static_cast<size_t>(j) * cols + col)
+                          : pack_status(kFlagPrefix, gen, 0u);
+        }
+        bool stalled = false;
+#pragma unroll
+        for (int i = 0; i < kLookbackWindow; ++i) {
+          if (!found_prefix && !stalled) {
+            const bool ready = (static_cast<uint32_t>(s[i] >> 32) & kGenMask) == gen && (s[i] >> 62) != 0;
+            if (ready) {
+              excl += static_cast<int>(static_cast<uint32_t>(s[i]));
+              found_prefix = (s[i] >> 62) == kFlagPrefix;
+              --next;
+              spins = 0;
+            } else {
+              stalled = true;
+            }
+          }
+        }
+        if (stalled) {
           if (++spins > a.spin_limit) {
             __hip_atomic_store(&a.ws->timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s = pack_status(kFlagPrefix, gen, 0u);
             break;
           }
           __builtin_amdgcn_s_sleep(2);
-          s = peek(theirs);
         }
-        excl += static_cast<int>(static_cast<uint32_t>(s));
-        if ((s >> 62) == kFlagPrefix) break;
       }
       publish(mine, pack_status(kFlagPrefix, gen, static_cast<uint32_t>(excl + total)));
     }
@@ -194,9 +245,10 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   // ---- position of every route inside its expert segment --------------------
   if (a.slot_rel != nullptr) {
 #pragma unroll
-    for (int c = 0; c < kMaxTopk; ++c) {
-      if (c < K) {
-        const int g = flat0 + (wave * K + c) * kWave + lane;
+    for (int c = 0; c < kChunksPerWave; ++c) {
+      const int chunk = wave * per_wave + c;
+      if (c < per_wave && chunk < num_chunks) {
+        const int g = flat0 + chunk * kWave + lane;
         if (g < flat_end) {
           const int e = my_e[c];
           a.slot_rel[g] = (e >= 0) ? col_excl[e] + my_hist[e] + my_pos[c] : -1;
@@ -232,18 +284,13 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
         a.num_tokens_per_rank[col - E] = cnt;
     }
     if (a.expert_offsets != nullptr) {
-      // Block-wide exclusive scan of the aligned counts; each thread owns a run
-      // of consecutive experts so that the scan order is the expert order.
-      const int per_thread = (E + kLayoutThreads - 1) / kLayoutThreads;
-      const int first = tid * per_thread;
+      // Block-wide exclusive scan of the aligned counts, one expert per thread
+      // (kMaxExperts <= kLayoutThreads), so the scan order is the expert order.
       const int align = a.expert_alignment;
       int local = 0;
-      for (int i = 0; i < per_thread; ++i) {
-        const int e = first + i;
-        if (e < E) {
-          const int cnt = col_excl[e] + col_total[e];
-          local += (cnt + align - 1) / align * align;
-        }
+      if (tid < E) {
+        const int cnt = col_excl[tid] + col_total[tid];
+        local = (cnt + align - 1) / align * align;
       }
       int incl = local;
 #pragma unroll
@@ -260,16 +307,9 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
         if (w < wave) base += wave_sums[w];
         grand += wave_sums[w];
       }
-      int* offs = hist;  // wave bases are no longer needed by this tile
-      __syncthreads();
-      for (int i = 0; i < per_thread; ++i) {
-        const int e = first + i;
-        if (e < E) {
-          offs[e] = base;
-          a.expert_offsets[e] = base;
-          const int cnt = col_excl[e] + col_total[e];
-          base += (cnt + align - 1) / align * align;
-        }
+      if (tid < E) {
+        offs[tid] = base;
+        a.expert_offsets[tid] = base;
       }
       if (tid == 0) {
         offs[E] = grand;
@@ -280,23 +320,10 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
         a.psum_rank_rows[tid] = offs[(tid + 1) * a.experts_per_rank];
     }
   }
-
-  // ---- hand the workspace back ready for the next launch --------------------
-  __syncthreads();
-  if (tid == 0) {
-    const uint32_t finished =
-        __hip_atomic_fetch_add(&a.ws->done, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    if (finished == static_cast<uint32_t>(a.num_tiles) - 1u) {
-      __hip_atomic_store(&a.ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(&a.ws->done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(&a.ws->generation, (gen + 1u) & kGenMask, __ATOMIC_RELEASE,
-                         __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
 }
 
 // Counts and flags only, accumulated with global atomics into zeroed outputs.
-__global__ __launch_bounds__(kLayoutThreads) void ep_layout_counts_kernel(
+__global__ __launch_bounds__(kCountsThreads) void ep_layout_counts_kernel(
     const int64_t* __restrict__ topk_idx, int* num_tokens_per_rank, int* num_tokens_per_expert,
     uint8_t* is_token_in_rank, int T, int K, int R, int E, int experts_per_rank, int expert_bits,
     int num_tiles) {
@@ -308,7 +335,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_counts_kernel(
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
 
-  for (int i = tid; i < E; i += kLayoutThreads) hist[i] = 0;
+  for (int i = tid; i < E; i += kCountsThreads) hist[i] = 0;
   if (tid < kMaxRanks) rank_cnt[tid] = 0;
   const int flat_end = T * K;
   for (int tile = static_cast<int>(blockIdx.x); tile < num_tiles; tile += static_cast<int>(gridDim.x)) {
@@ -339,7 +366,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_counts_kernel(
     __syncthreads();
   }
   __syncthreads();
-  for (int i = tid; i < E; i += kLayoutThreads)
+  for (int i = tid; i < E; i += kCountsThreads)
     if (hist[i] != 0) atomicAdd(&num_tokens_per_expert[i], hist[i]);
   if (tid < R && rank_cnt[tid] != 0) atomicAdd(&num_tokens_per_rank[tid], rank_cnt[tid]);
 }
@@ -369,10 +396,11 @@ hipError_t launch_fill_u32(uint32_t* dst, size_t count, uint32_t value, hipStrea
 }
 
 hipError_t launch_layout_fused(const LayoutArgs& a, hipStream_t stream) {
-  const int cols = a.num_experts + a.num_ranks;
-  const size_t lds = sizeof(int) * (static_cast<size_t>(kLayoutWaves) * a.num_experts + 2 * cols +
-                                    kMaxRanks + kLayoutWaves + 4) +
-                     sizeof(uint64_t) * kTileTokens;
+  static_assert(kMaxExperts <= kLayoutThreads, "the offset scan takes one expert per thread");
+  const int E = a.num_experts;
+  const int cols = E + a.num_ranks;
+  const size_t lds = sizeof(int) * (2 * static_cast<size_t>(cols) + kMaxRanks + kLayoutWaves + 4 + E + 2 + (E & 1)) +
+                     sizeof(uint64_t) * kTileTokens + sizeof(uint16_t) * (static_cast<size_t>(kLayoutWaves) * E + 2);
   hipLaunchKernelGGL(ep_layout_fused_kernel, dim3(a.num_tiles), dim3(kLayoutThreads), lds, stream, a);
   return hipGetLastError();
 }
@@ -392,7 +420,7 @@ hipError_t launch_layout_counts(const int64_t* topk_idx, int* num_tokens_per_ran
   const int grid = num_tiles < 1024 ? num_tiles : 1024;
   const size_t lds = sizeof(int) * (num_experts + kMaxRanks + (num_experts & 1)) +
                      sizeof(uint64_t) * kTileTokens;
-  hipLaunchKernelGGL(ep_layout_counts_kernel, dim3(grid), dim3(kLayoutThreads), lds, stream, topk_idx,
+  hipLaunchKernelGGL(ep_layout_counts_kernel, dim3(grid), dim3(kCountsThreads), lds, stream, topk_idx,
                      num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, num_tokens, num_topk,
                      num_ranks, num_experts, num_experts / num_ranks, expert_bits, num_tiles);
   return hipGetLastError();

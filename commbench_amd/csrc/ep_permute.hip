@@ -36,7 +36,7 @@ __global__ __launch_bounds__(kPermuteThreads) void ep_permute_kernel(const Permu
 #pragma unroll
   for (int u = 0; u < kBatchVecs; ++u) {
     const int v = v0 + u * kWave;
-    if (v < a.row_vecs) buf[u] = __builtin_nontemporal_load(src + v);
+    if (v < a.row_vecs) buf[u] = src[v];
   }
 
   // Lane k < K resolves slot k of the token.
