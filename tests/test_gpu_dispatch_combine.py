@@ -163,6 +163,30 @@ def test_combine_every_topk_with_biases(oracle, K):
         assert worst == 0, "same fma chain on both sides: expected bit-exact"
 
 
+@pytest.mark.parametrize("shape", [(4099, 3, 1032), (6000, 8, 2048), (4096, 1, 1024), (9001, 5, 1280)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_combine_large_token_counts_use_the_staged_schedule(oracle, shape):
+    """>= 16 tokens per compute unit and rows >= 2 KiB take the persistent LDS-staged schedule:
+    ragged token ranges, ragged last vectors, masks, weights on/off and both biases."""
+    T, K, H = shape
+    print(f"shape {shape}", flush=True)
+    rng = np.random.default_rng(T + K)
+    E, R = 64, 8
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    topk_np[rng.random((T, K)) < 0.1] = -1
+    topk_np[5] = -1                                   # a token with no routes at all
+    w_np = wl.softmax_gates(rng, T, K)
+    _, per_expert, _ = oracle.layout(topk_np, R, E)
+    off, _ = oracle.expert_offsets(per_expert, R, 1)
+    _, slot_map, _, _ = oracle.slot_maps(topk_np, E, off)
+    y = wl.bf16_normal(rng, int(off[-1]), H).to(gu.DEV)
+    b0, b1 = wl.bf16_normal(rng, T, H), wl.bf16_normal(rng, T, H)
+    sm = torch.from_numpy(slot_map).to(gu.DEV)
+    for weights, biases in ((w_np, (None, None)), (None, (b0, b1))):
+        got, want, worst = combine_and_check(oracle, y, sm, weights, slot_map, biases)
+        assert worst == 0
+
+
 def test_combine_integer_payload_is_exact(oracle):
     rng = np.random.default_rng(21)
     T, K, E, R, H = 500, 8, 64, 8, 256
