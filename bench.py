@@ -228,7 +228,12 @@ def main():
         ev[3].record()
     torch.cuda.synchronize()
 
-    names = ["ep_layout_fused_kernel", "ep_permute_kernel", "ep_combine_kernel"]
+    # Kernel symbols as rocprofv3 reports them; the combine schedule depends on the shape
+    # (persistent LDS-staged kernel from 16 tokens per compute unit and 2 KiB rows upwards).
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    staged = T >= 16 * cus and 2048 <= cfg.hidden * 2 <= 160 * 1024
+    names = ["ep_layout_fused_kernel", "ep_permute_kernel",
+             "ep_combine_staged_kernel" if staged else "ep_combine_kernel"]
     kernel_us = {n: sum(ev[i].elapsed_time(ev[i + 1]) for ev in marks) * 1e3 / args.steps
                  for i, n in enumerate(names)}
     kernel_bytes = dict(zip(names, (wk.bytes["layout"], wk.bytes["dispatch"], wk.bytes["combine"])))

@@ -1,0 +1,316 @@
+// Self-checking executable in the reference's own style: a correctness phase against the CPU
+// checker, then a benchmark phase, then exactly one JSON object on stdout; exit code 0 <=> PASS
+// (datasets/readme.md:127-167 of the reference).  It drives the C++ surface of include/mi_ep.hpp
+// the way the reference's main() drives its classes
+// (datasets/example042_deepep_dispatch_layout/nv/empty_deepep_dispatch_layout.cu:391-427):
+// the same 13 correctness cases and 7 benchmark cases, 20 warm-up + 100 timed launches between two
+// events, Mtokens/s = tokens / microsecond.  Added beyond the reference: the fused layout on the
+// same cases, the notify example's channel-prefix cases (example047 .cu:599-610) and one
+// dispatch -> combine round trip.
+//
+// Test code: links the CPU checker (oracle/libep_oracle.so) as well as libmi_ep.so.
+#include <algorithm>
+#include <cstring>
+#include <iomanip>
+#include <iostream>
+#include <string>
+#include <vector>
+
+#include "mi_ep.hpp"
+
+extern "C" {
+int ep_oracle_layout(const int64_t*, int, int, int, int, int*, int*, uint8_t*);
+int ep_oracle_expert_offsets(const int*, int, int, int, int*, int*);
+int ep_oracle_slot_maps(const int64_t*, int, int, int, const int*, int*, int*, int*, int*, int*);
+int ep_oracle_channel_prefix(const uint8_t*, int, int, int, int*);
+int ep_oracle_permute(const void*, int, const float*, int, const int64_t*, const float*, int, const int*,
+                      const int*, int, void*, float*, int64_t*, float*, int);
+int ep_oracle_combine(const uint16_t*, const int*, const float*, const uint16_t*, const uint16_t*, int, int,
+                      int, uint16_t*, int);
+uint16_t ep_oracle_f32_to_bf16(float);
+}
+
+namespace {
+
+using mi_ep::TopkIdx;
+
+enum Pattern { kSpread = 0, kRankSweep = 1, kSameRank = 2 };
+const char* pattern_name(int p) { return p == kRankSweep ? "rank_sweep" : p == kSameRank ? "same_rank" : "spread"; }
+
+struct Case { int tokens, topk, ranks, experts, pattern; };
+
+// The reference's closed-form routing tables (example042 .cu:178-206).
+std::vector<TopkIdx> make_topk(const Case& c) {
+  std::vector<TopkIdx> idx(static_cast<size_t>(c.tokens) * c.topk);
+  const int per_rank = c.experts / c.ranks;
+  for (int t = 0; t < c.tokens; ++t)
+    for (int k = 0; k < c.topk; ++k) {
+      int e;
+      switch (c.pattern) {
+        case kRankSweep: e = ((t + k) % c.ranks) * per_rank + (5 * t + 3 * k) % per_rank; break;
+        case kSameRank: e = ((3 * t + c.topk) % c.ranks) * per_rank + (t + 7 * k) % per_rank; break;
+        default: e = (17 * t + 31 * k + c.ranks) % c.experts; break;
+      }
+      idx[static_cast<size_t>(t) * c.topk + k] = e;
+    }
+  return idx;
+}
+
+template <class T>
+struct DeviceArray {
+  T* p = nullptr;
+  size_t n = 0;
+  explicit DeviceArray(size_t count) : n(count) { MI_EP_HIP_CHECK(hipMalloc(&p, std::max<size_t>(count, 1) * sizeof(T))); }
+  ~DeviceArray() { (void)hipFree(p); }
+  void upload(const std::vector<T>& h) { MI_EP_HIP_CHECK(hipMemcpy(p, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice)); }
+  std::vector<T> download(size_t count) const {
+    std::vector<T> h(count);
+    MI_EP_HIP_CHECK(hipMemcpy(h.data(), p, count * sizeof(T), hipMemcpyDeviceToHost));
+    return h;
+  }
+  void fill_bytes(int v) { MI_EP_HIP_CHECK(hipMemset(p, v, std::max<size_t>(n, 1) * sizeof(T))); }
+};
+
+struct HostLayout {
+  std::vector<int> per_rank, per_expert, offsets, psum, slot_rel, slot_map, src_map, src_k;
+  std::vector<uint8_t> flags;
+};
+
+HostLayout host_layout(const Case& c, const std::vector<TopkIdx>& idx, int align) {
+  HostLayout h;
+  h.per_rank.resize(c.ranks);
+  h.per_expert.resize(c.experts);
+  h.flags.resize(static_cast<size_t>(c.tokens) * c.ranks);
+  ep_oracle_layout(idx.data(), c.tokens, c.topk, c.ranks, c.experts, h.per_rank.data(), h.per_expert.data(), h.flags.data());
+  h.offsets.resize(c.experts + 1);
+  h.psum.resize(c.ranks);
+  ep_oracle_expert_offsets(h.per_expert.data(), c.experts, c.ranks, align, h.offsets.data(), h.psum.data());
+  const size_t tk = static_cast<size_t>(c.tokens) * c.topk;
+  h.slot_rel.resize(tk);
+  h.slot_map.resize(tk);
+  h.src_map.resize(h.offsets.back());
+  h.src_k.resize(h.offsets.back());
+  std::vector<int> fill(c.experts);
+  ep_oracle_slot_maps(idx.data(), c.tokens, c.topk, c.experts, h.offsets.data(), h.slot_rel.data(), h.slot_map.data(),
+                      h.src_map.data(), h.src_k.data(), fill.data());
+  return h;
+}
+
+// Counts + flags through DeepepDispatchLayout, as the reference's runCorrectnessCase (:236-295).
+bool check_counts_surface(const Case& c) {
+  const std::vector<TopkIdx> idx = make_topk(c);
+  const HostLayout ref = host_layout(c, idx, 1);
+  DeviceArray<TopkIdx> d_idx(idx.size());
+  DeviceArray<int> d_rank(c.ranks), d_expert(c.experts);
+  DeviceArray<bool> d_flags(static_cast<size_t>(c.tokens) * c.ranks);
+  d_idx.upload(idx);
+  d_rank.fill_bytes(0);
+  d_expert.fill_bytes(0);
+  d_flags.fill_bytes(0);
+  mi_ep::DeepepDispatchLayout layout(c.tokens, c.topk, c.ranks, c.experts);
+  layout.compute(d_idx.p, d_rank.p, d_expert.p, d_flags.p);
+  layout.compute(d_idx.p, d_rank.p, d_expert.p, d_flags.p);  // relaunch without re-zeroing (:313-329)
+  MI_EP_HIP_CHECK(hipDeviceSynchronize());
+  bool ok = d_rank.download(c.ranks) == ref.per_rank && d_expert.download(c.experts) == ref.per_expert;
+  const std::vector<bool> dummy;
+  std::vector<uint8_t> got(ref.flags.size());
+  MI_EP_HIP_CHECK(hipMemcpy(got.data(), d_flags.p, got.size(), hipMemcpyDeviceToHost));
+  for (size_t i = 0; i < got.size(); ++i) ok = ok && ((got[i] != 0) == (ref.flags[i] != 0));
+  return ok;
+}
+
+// Fused layout through ExpertParallelBuffer: everything the counts surface gives plus offsets,
+// partition rows, channel prefixes and per-route positions, bit-exact.
+bool check_fused_surface(const Case& c, int align, int channels) {
+  const std::vector<TopkIdx> idx = make_topk(c);
+  const HostLayout ref = host_layout(c, idx, align);
+  DeviceArray<TopkIdx> d_idx(idx.size());
+  d_idx.upload(idx);
+  mi_ep::ExpertParallelBuffer buf(c.tokens, c.topk, c.experts, c.ranks, align, channels);
+  const mi_ep::DispatchHandle& h = buf.get_dispatch_layout(d_idx.p, c.tokens);
+  buf.check_status();
+  auto pull = [](const int* p, size_t n) {
+    std::vector<int> v(n);
+    MI_EP_HIP_CHECK(hipMemcpy(v.data(), p, n * sizeof(int), hipMemcpyDeviceToHost));
+    return v;
+  };
+  bool ok = pull(h.num_tokens_per_rank, c.ranks) == ref.per_rank && pull(h.num_tokens_per_expert, c.experts) == ref.per_expert &&
+            pull(h.expert_offsets, c.experts + 1) == ref.offsets && pull(h.psum_rank_rows, c.ranks) == ref.psum &&
+            pull(h.slot_rel, ref.slot_rel.size()) == ref.slot_rel;
+  std::vector<uint8_t> flags(ref.flags.size());
+  MI_EP_HIP_CHECK(hipMemcpy(flags.data(), h.is_token_in_rank, flags.size(), hipMemcpyDeviceToHost));
+  ok = ok && flags == ref.flags;
+  if (channels > 0) {
+    std::vector<int> want(static_cast<size_t>(c.ranks) * channels);
+    ep_oracle_channel_prefix(ref.flags.data(), c.tokens, c.ranks, channels, want.data());
+    ok = ok && pull(h.channel_prefix_matrix, want.size()) == want;
+  }
+  return ok;
+}
+
+// The notify example's inputs (example047 .cu:189-193,437-447) for source rank 0: two
+// destinations per token, one expert per rank; C = min(16, max(4, 2R)).
+bool check_notify_case(int tokens, int ranks) {
+  Case c{tokens, std::min(2, ranks), ranks, ranks, kSpread};
+  std::vector<TopkIdx> idx(static_cast<size_t>(tokens) * c.topk);
+  for (int t = 0; t < tokens; ++t)
+    for (int s = 0; s < c.topk; ++s) idx[static_cast<size_t>(t) * c.topk + s] = (t + s) % ranks;
+  const int channels = std::min(16, std::max(4, 2 * ranks));
+  const HostLayout ref = host_layout(c, idx, 1);
+  std::vector<int> want(static_cast<size_t>(ranks) * channels);
+  ep_oracle_channel_prefix(ref.flags.data(), tokens, ranks, channels, want.data());
+  DeviceArray<TopkIdx> d_idx(idx.size());
+  d_idx.upload(idx);
+  mi_ep::ExpertParallelBuffer buf(tokens, c.topk, ranks, ranks, 1, channels);
+  const mi_ep::DispatchHandle& h = buf.get_dispatch_layout(d_idx.p, tokens);
+  buf.check_status();
+  std::vector<int> got(want.size());
+  MI_EP_HIP_CHECK(hipMemcpy(got.data(), h.channel_prefix_matrix, got.size() * sizeof(int), hipMemcpyDeviceToHost));
+  return got == want;
+}
+
+// Dispatch -> identity experts -> weighted combine on a small bf16 case, against the checker.
+bool check_round_trip() {
+  Case c{517, 8, 8, 64, kRankSweep};
+  const int hidden = 1032, row_bytes = hidden * 2;
+  std::vector<TopkIdx> idx = make_topk(c);
+  for (size_t i = 0; i < idx.size(); i += 13) idx[i] = -1;  // masked slots
+  std::vector<float> w(idx.size());
+  for (size_t i = 0; i < w.size(); ++i) w[i] = 0.03125f * static_cast<float>(1 + (i * 7) % 11);
+  std::vector<uint16_t> x(static_cast<size_t>(c.tokens) * hidden);
+  for (size_t i = 0; i < x.size(); ++i) x[i] = ep_oracle_f32_to_bf16(static_cast<float>(static_cast<int>((i * 2654435761u) >> 20 & 1023) - 512) / 64.0f);
+  const HostLayout ref = host_layout(c, idx, 1);
+  const int rows = ref.offsets.back();
+  std::vector<uint16_t> want_recv(static_cast<size_t>(rows) * hidden), want_out(x.size());
+  std::vector<int64_t> want_idx(rows);
+  std::vector<float> want_w(rows);
+  ep_oracle_permute(x.data(), row_bytes, nullptr, 0, idx.data(), w.data(), c.topk, ref.src_map.data(), ref.src_k.data(),
+                    rows, want_recv.data(), nullptr, want_idx.data(), want_w.data(), 1);
+  ep_oracle_combine(want_recv.data(), ref.slot_map.data(), w.data(), nullptr, nullptr, c.tokens, c.topk, hidden,
+                    want_out.data(), 1);
+
+  DeviceArray<TopkIdx> d_idx(idx.size());
+  DeviceArray<float> d_w(w.size());
+  DeviceArray<uint16_t> d_x(x.size()), d_out(x.size());
+  d_idx.upload(idx);
+  d_w.upload(w);
+  d_x.upload(x);
+  mi_ep::ExpertParallelBuffer buf(c.tokens, c.topk, c.experts, c.ranks);
+  DeviceArray<uint16_t> d_recv(static_cast<size_t>(buf.capacity_rows()) * hidden);
+  const mi_ep::DispatchHandle& h = buf.dispatch(d_x.p, nullptr, d_idx.p, d_w.p, c.tokens, row_bytes, 0, d_recv.p, nullptr);
+  buf.combine(d_recv.p, d_w.p, nullptr, nullptr, hidden, d_out.p);
+  buf.check_status();
+  bool ok = d_recv.download(want_recv.size()) == want_recv;
+  std::vector<int> got_map(ref.slot_map.size()), got_src(rows);
+  MI_EP_HIP_CHECK(hipMemcpy(got_map.data(), h.slot_map, got_map.size() * sizeof(int), hipMemcpyDeviceToHost));
+  MI_EP_HIP_CHECK(hipMemcpy(got_src.data(), h.recv_src_map, got_src.size() * sizeof(int), hipMemcpyDeviceToHost));
+  ok = ok && got_map == ref.slot_map && got_src == ref.src_map;
+  ok = ok && d_out.download(want_out.size()) == want_out;  // same fma chain: bit-exact
+  return ok;
+}
+
+struct MetricRow {
+  std::string surface;
+  Case c;
+  double latency_us = 0.0, mtokens_per_s = 0.0;
+};
+
+template <class Launch>
+MetricRow time_launches(const std::string& surface, const Case& c, Launch launch) {
+  const int warmup_iters = 20, bench_iters = 100;
+  for (int i = 0; i < warmup_iters; ++i) launch();
+  MI_EP_HIP_CHECK(hipDeviceSynchronize());
+  hipEvent_t start, stop;
+  MI_EP_HIP_CHECK(hipEventCreate(&start));
+  MI_EP_HIP_CHECK(hipEventCreate(&stop));
+  MI_EP_HIP_CHECK(hipEventRecord(start));
+  for (int i = 0; i < bench_iters; ++i) launch();
+  MI_EP_HIP_CHECK(hipEventRecord(stop));
+  MI_EP_HIP_CHECK(hipEventSynchronize(stop));
+  float ms = 0.0f;
+  MI_EP_HIP_CHECK(hipEventElapsedTime(&ms, start, stop));
+  MI_EP_HIP_CHECK(hipEventDestroy(start));
+  MI_EP_HIP_CHECK(hipEventDestroy(stop));
+  MetricRow row{surface, c};
+  row.latency_us = static_cast<double>(ms) * 1000.0 / bench_iters;
+  row.mtokens_per_s = row.latency_us > 0.0 ? c.tokens / row.latency_us : 0.0;
+  return row;
+}
+
+void benchmark_case(const Case& c, std::vector<MetricRow>* rows) {
+  const std::vector<TopkIdx> idx = make_topk(c);
+  DeviceArray<TopkIdx> d_idx(idx.size());
+  DeviceArray<int> d_rank(c.ranks), d_expert(c.experts);
+  DeviceArray<bool> d_flags(static_cast<size_t>(c.tokens) * c.ranks);
+  d_idx.upload(idx);
+  mi_ep::DeepepDispatchLayout layout(c.tokens, c.topk, c.ranks, c.experts);
+  rows->push_back(time_launches("get_dispatch_layout", c, [&] { layout.compute(d_idx.p, d_rank.p, d_expert.p, d_flags.p); }));
+  mi_ep::ExpertParallelBuffer buf(c.tokens, c.topk, c.experts, c.ranks);
+  rows->push_back(time_launches("fused_layout", c, [&] { buf.get_dispatch_layout(d_idx.p, c.tokens); }));
+  buf.check_status();
+}
+
+void print_json(bool pass, const std::vector<MetricRow>& rows) {
+  std::cout << std::fixed << std::setprecision(3);
+  std::cout << "{\n  \"Correctness\": \"" << (pass ? "PASS" : "FAIL") << "\",\n";
+  std::cout << "  \"data_size_unit\": \"tokens\",\n  \"throughput_unit\": \"Mtokens/s\",\n  \"latency_unit\": \"us\",\n";
+  std::cout << "  \"metrics\": [\n";
+  for (size_t i = 0; i < rows.size(); ++i) {
+    const MetricRow& r = rows[i];
+    std::cout << "    {\"surface\": \"" << r.surface << "\", \"data_size\": " << r.c.tokens << ", \"num_topk\": " << r.c.topk
+              << ", \"num_ranks\": " << r.c.ranks << ", \"num_experts\": " << r.c.experts << ", \"pattern\": \""
+              << pattern_name(r.c.pattern) << "\", \"throughput_avg\": " << r.mtokens_per_s
+              << ", \"latency_avg\": " << r.latency_us << "}" << (i + 1 != rows.size() ? "," : "") << "\n";
+  }
+  std::cout << "  ]\n}\n";
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  const bool skip_bench = argc > 1 && std::string(argv[1]) == "--skip-perf-test";
+  int device_count = 0;
+  if (hipGetDeviceCount(&device_count) != hipSuccess || device_count <= 0) {
+    std::cout << "{\"Correctness\": \"SKIP\", \"reason\": \"no HIP device available\"}\n";
+    return 0;
+  }
+  MI_EP_HIP_CHECK(hipSetDevice(0));
+
+  std::vector<Case> cases = {{257, 1, 1, 4, kSpread}};
+  for (int r : {2, 4, 8}) {
+    cases.push_back({257, 1, r, 4 * r, kSpread});
+    cases.push_back({1024, 2, r, 4 * r, kSpread});
+    cases.push_back({4096, 4, r, 4 * r, kRankSweep});
+    cases.push_back({4096, 8, r, 4 * r, kSameRank});
+  }
+  bool pass = true;
+  for (const Case& c : cases) {
+    const bool a = check_counts_surface(c);
+    const bool b = check_fused_surface(c, 1, 2 * c.ranks) && check_fused_surface(c, 128, 0);
+    if (!a || !b)
+      std::cerr << "FAIL layout case T=" << c.tokens << " K=" << c.topk << " R=" << c.ranks << " E=" << c.experts << " "
+                << pattern_name(c.pattern) << " counts=" << a << " fused=" << b << "\n";
+    pass = pass && a && b;
+  }
+  for (int r : {2, 4, 8})
+    for (int t : {7, 4096, 4097}) {
+      const bool ok = check_notify_case(t, r);
+      if (!ok) std::cerr << "FAIL notify case T=" << t << " R=" << r << "\n";
+      pass = pass && ok;
+    }
+  {
+    const bool ok = check_round_trip();
+    if (!ok) std::cerr << "FAIL dispatch/combine round trip\n";
+    pass = pass && ok;
+  }
+
+  std::vector<MetricRow> rows;
+  if (!skip_bench) {
+    for (int tokens : {1024, 4096, 16384, 65536}) benchmark_case({tokens, 2, 8, 32, kSpread}, &rows);
+    benchmark_case({65536, 4, 8, 32, kRankSweep}, &rows);
+    benchmark_case({65536, 8, 8, 32, kSameRank}, &rows);
+    benchmark_case({65536, 2, 4, 32, kSpread}, &rows);
+  }
+  print_json(pass, rows);
+  return pass ? 0 : 1;
+}

@@ -1,0 +1,38 @@
+"""Runs the C++ self-checking harness (tests/cpp/ep_selftest), which drives include/mi_ep.hpp the
+way the reference's main() drives its classes and prints the reference's one-JSON-object protocol."""
+import json
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BINARY = os.path.join(ROOT, "tests", "cpp", "ep_selftest")
+
+
+@pytest.mark.gpu
+def test_selftest_binary_passes():
+    assert os.path.exists(BINARY), "build with `make -C tests/cpp` (done by __graft_entry__.build())"
+    proc = subprocess.run([BINARY], capture_output=True, text=True, timeout=300)
+    print(proc.stderr)
+    report = json.loads(proc.stdout)
+    assert report["Correctness"] == "PASS" and proc.returncode == 0
+    rows = report["metrics"]
+    assert len(rows) == 14                     # the reference's 7 benchmark cases on both surfaces
+    assert {r["surface"] for r in rows} == {"get_dispatch_layout", "fused_layout"}
+    assert all(r["throughput_avg"] > 0 for r in rows)
+    out_dir = os.path.join(ROOT, "gpurun_out")       # kept when the run's outputs are collected
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "selftest.json"), "w") as f:
+            f.write(proc.stdout)
+
+
+def test_selftest_binary_skips_without_a_device():
+    """Same protocol as the reference when no device is present: SKIP, exit code 0."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    if not os.path.exists(BINARY):
+        pytest.skip("binary not built")
+    proc = subprocess.run([BINARY], capture_output=True, text=True, timeout=60)
+    assert proc.returncode == 0 and json.loads(proc.stdout)["Correctness"] == "SKIP"
