@@ -39,7 +39,7 @@ constexpr uint32_t kFlagAggregate = 1;
 constexpr uint32_t kFlagPrefix = 2;
 constexpr uint32_t kGenMask = 0x3fffffffu;
 constexpr int kLookbackWindow = 32;
-constexpr int kCountsThreads = 256;  // the counts-only kernel: one token per thread, 4 waves
+constexpr int kCountsThreads = 1024;  // the counts-only kernel: one token per thread, 16 waves
 
 __device__ __forceinline__ uint64_t pack_status(uint32_t flag, uint32_t gen, uint32_t value) {
   return (static_cast<uint64_t>(flag) << 62) | (static_cast<uint64_t>(gen & kGenMask) << 32) |
@@ -322,15 +322,17 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   }
 }
 
-// Counts and flags only, accumulated with global atomics into zeroed outputs.
+// Counts and flags only.  One token per thread, 1024 tokens per workgroup pass; totals are
+// accumulated with global atomics into zeroed outputs, or stored directly when one
+// workgroup covers every token.
 __global__ __launch_bounds__(kCountsThreads) void ep_layout_counts_kernel(
     const int64_t* __restrict__ topk_idx, int* num_tokens_per_rank, int* num_tokens_per_expert,
     uint8_t* is_token_in_rank, int T, int K, int R, int E, int experts_per_rank, int expert_bits,
-    int num_tiles) {
+    int num_tiles, int single_workgroup) {
   extern __shared__ int smem[];
   int* hist = smem;                // [E]
   int* rank_cnt = hist + E;        // [kMaxRanks]
-  uint64_t* tok_flags = reinterpret_cast<uint64_t*>(rank_cnt + kMaxRanks + (E & 1));  // [kTileTokens]
+  uint64_t* tok_flags = reinterpret_cast<uint64_t*>(rank_cnt + kMaxRanks + (E & 1));  // [kCountsThreads]
   const int tid = static_cast<int>(threadIdx.x);
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
@@ -341,18 +343,26 @@ __global__ __launch_bounds__(kCountsThreads) void ep_layout_counts_kernel(
   for (int tile = static_cast<int>(blockIdx.x); tile < num_tiles; tile += static_cast<int>(gridDim.x)) {
     tok_flags[tid] = 0;
     __syncthreads();
-    const int t0 = tile * kTileTokens;
+    const int t0 = tile * kCountsThreads;
     const int flat0 = t0 * K;
-    for (int c = 0; c < K; ++c) {
-      const int local = (wave * K + c) * kWave + lane;
-      const int g = flat0 + local;
-      const int64_t e64 = (g < flat_end) ? topk_idx[g] : -1;
-      const bool valid = e64 >= 0 && e64 < static_cast<int64_t>(E);
-      const int e = valid ? static_cast<int>(e64) : 0;
-      const uint64_t same = match_expert(valid, e, expert_bits);
-      if (valid) {
-        if ((same & lanes_below(lane)) == 0) atomicAdd(&hist[e], __popcll(same));
-        reinterpret_cast<uint8_t*>(tok_flags + local / K)[e / experts_per_rank] = 1;
+    int64_t raw[kMaxTopk];  // every chunk's load is in flight before the first ballot
+#pragma unroll
+    for (int c = 0; c < kMaxTopk; ++c) {
+      const int g = flat0 + (wave * K + c) * kWave + lane;
+      raw[c] = (c < K && g < flat_end) ? topk_idx[g] : -1;
+    }
+#pragma unroll
+    for (int c = 0; c < kMaxTopk; ++c) {
+      if (c < K) {
+        const int local = (wave * K + c) * kWave + lane;
+        const int64_t e64 = raw[c];
+        const bool valid = e64 >= 0 && e64 < static_cast<int64_t>(E);
+        const int e = valid ? static_cast<int>(e64) : 0;
+        const uint64_t same = match_expert(valid, e, expert_bits);
+        if (valid) {
+          if ((same & lanes_below(lane)) == 0) atomicAdd(&hist[e], __popcll(same));
+          reinterpret_cast<uint8_t*>(tok_flags + local / K)[e / experts_per_rank] = 1;
+        }
       }
     }
     __syncthreads();
@@ -366,6 +376,12 @@ __global__ __launch_bounds__(kCountsThreads) void ep_layout_counts_kernel(
     __syncthreads();
   }
   __syncthreads();
+  if (single_workgroup) {
+    // The only workgroup has seen every token: plain stores, no zeroing pass needed.
+    for (int i = tid; i < E; i += kCountsThreads) num_tokens_per_expert[i] = hist[i];
+    if (tid < R) num_tokens_per_rank[tid] = rank_cnt[tid];
+    return;
+  }
   for (int i = tid; i < E; i += kCountsThreads)
     if (hist[i] != 0) atomicAdd(&num_tokens_per_expert[i], hist[i]);
   if (tid < R && rank_cnt[tid] != 0) atomicAdd(&num_tokens_per_rank[tid], rank_cnt[tid]);
@@ -409,20 +425,26 @@ hipError_t launch_layout_counts(const int64_t* topk_idx, int* num_tokens_per_ran
                                 int* num_tokens_per_expert, uint8_t* is_token_in_rank,
                                 int num_tokens, int num_topk, int num_ranks, int num_experts,
                                 hipStream_t stream) {
-  const int n = num_experts > num_ranks ? num_experts : num_ranks;
-  hipLaunchKernelGGL(ep_zero_counts_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
-                     num_tokens_per_expert, num_experts, num_tokens_per_rank, num_ranks);
-  hipError_t err = hipGetLastError();
-  if (err != hipSuccess || num_tokens == 0) return err;
-  const int num_tiles = (num_tokens + kTileTokens - 1) / kTileTokens;
+  const int num_tiles = (num_tokens + kCountsThreads - 1) / kCountsThreads;
+  // Up to 1024 tokens one workgroup sees everything and stores the totals itself: one
+  // launch instead of zero + accumulate, which is what matters at these sizes.
+  const bool single = num_tiles == 1;
+  if (!single) {
+    const int n = num_experts > num_ranks ? num_experts : num_ranks;
+    hipLaunchKernelGGL(ep_zero_counts_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
+                       num_tokens_per_expert, num_experts, num_tokens_per_rank, num_ranks);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess || num_tokens == 0) return err;
+  }
   int expert_bits = 1;
   while ((1 << expert_bits) < num_experts) ++expert_bits;
-  const int grid = num_tiles < 1024 ? num_tiles : 1024;
+  const int grid = single ? 1 : (num_tiles < 1024 ? num_tiles : 1024);
   const size_t lds = sizeof(int) * (num_experts + kMaxRanks + (num_experts & 1)) +
-                     sizeof(uint64_t) * kTileTokens;
+                     sizeof(uint64_t) * kCountsThreads;
   hipLaunchKernelGGL(ep_layout_counts_kernel, dim3(grid), dim3(kCountsThreads), lds, stream, topk_idx,
                      num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, num_tokens, num_topk,
-                     num_ranks, num_experts, num_experts / num_ranks, expert_bits, num_tiles);
+                     num_ranks, num_experts, num_experts / num_ranks, expert_bits, num_tiles,
+                     single ? 1 : 0);
   return hipGetLastError();
 }
 

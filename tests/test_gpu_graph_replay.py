@@ -1,0 +1,90 @@
+"""The three calls captured in one HIP graph: every replay must equal the eager result, also after
+the inputs changed in place and with eager work and synchronisations between replays (the layout
+kernel's workspace hands itself over from launch to launch without any clearing node)."""
+import numpy as np
+import pytest
+import torch
+
+from commbench_amd import _lib, ops
+from commbench_amd import workloads as wl
+
+from . import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+
+
+def test_graph_replays_match_eager(oracle):
+    T, K, E, R, H = 3000, 8, 64, 8, 1024
+    rng = np.random.default_rng(12)
+    lib = _lib.load()
+    dev = gu.DEV
+    topk = torch.empty((T, K), dtype=torch.int64, device=dev)
+    w = torch.empty((T, K), dtype=torch.float32, device=dev)
+    x = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    cap = T * K
+    i32 = dict(dtype=torch.int32, device=dev)
+    per_rank, per_expert = torch.empty(R, **i32), torch.empty(E, **i32)
+    in_rank = torch.empty((T, R), dtype=torch.bool, device=dev)
+    off, psum = torch.empty(E + 1, **i32), torch.empty(R, **i32)
+    slot_rel, slot_map = torch.empty((T, K), **i32), torch.empty((T, K), **i32)
+    src_map = torch.empty(cap, **i32)
+    recv_idx = torch.empty(cap, dtype=torch.int64, device=dev)
+    recv_w = torch.empty(cap, dtype=torch.float32, device=dev)
+    recv_x = torch.empty((cap, H), dtype=torch.bfloat16, device=dev)
+    out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    ws_bytes = lib.mi_ep_workspace_bytes(T, K, E, R)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    _lib.check(lib.mi_ep_workspace_init(ws.data_ptr(), ws_bytes, torch.cuda.current_stream().cuda_stream), "init")
+
+    def step(stream):
+        _lib.check(lib.mi_ep_dispatch_layout(
+            topk.data_ptr(), T, K, R, E, 1, 0, per_rank.data_ptr(), per_expert.data_ptr(),
+            in_rank.data_ptr(), off.data_ptr(), psum.data_ptr(), None, slot_rel.data_ptr(),
+            ws.data_ptr(), ws_bytes, stream), "layout")
+        _lib.check(lib.mi_ep_dispatch(
+            x.data_ptr(), None, topk.data_ptr(), w.data_ptr(), off.data_ptr(), slot_rel.data_ptr(),
+            per_expert.data_ptr(), T, K, E, 1, H * 2, 0, recv_x.data_ptr(), None, src_map.data_ptr(),
+            recv_idx.data_ptr(), recv_w.data_ptr(), slot_map.data_ptr(), cap, stream), "dispatch")
+        _lib.check(lib.mi_ep_combine(
+            recv_x.data_ptr(), slot_map.data_ptr(), w.data_ptr(), None, None, None, T, K, H,
+            out.data_ptr(), None, stream), "combine")
+
+    def load_inputs(seed):
+        r = np.random.default_rng(seed)
+        t = wl.zipf_distinct_topk(r, T, E, K, 1.2)
+        t[r.random((T, K)) < 0.05] = -1
+        topk.copy_(torch.from_numpy(t))
+        w.copy_(torch.from_numpy(wl.softmax_gates(r, T, K)))
+        x.copy_(wl.bf16_normal(r, T, H))
+        return t
+
+    def snapshot():
+        torch.cuda.synchronize()
+        rows = int(off[-1].item())
+        return (per_expert.cpu().numpy().copy(), slot_map.cpu().numpy().copy(),
+                gu.bf16_bits(recv_x[:rows]).copy(), gu.bf16_bits(out).copy())
+
+    load_inputs(0)
+    step(torch.cuda.current_stream().cuda_stream)          # eager warm-up before capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+
+    for seed in (1, 2, 3, 4):
+        t_np = load_inputs(seed)
+        step(torch.cuda.current_stream().cuda_stream)      # eager
+        eager = snapshot()
+        for buf in (per_expert, slot_map, recv_x, out):
+            buf.view(torch.uint8).fill_(0x5A)               # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        replayed = snapshot()
+        for a, b in zip(eager, replayed):
+            np.testing.assert_array_equal(a, b)
+        _, want_expert, _ = oracle.layout(t_np, R, E)
+        np.testing.assert_array_equal(replayed[0], want_expert)
+    _lib.check(lib.mi_ep_workspace_status(ws.data_ptr(), torch.cuda.current_stream().cuda_stream), "status")
