@@ -196,6 +196,30 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
   return status_of(e);
 }
 
+int mi_ep_dispatch_cached(const void* x, const float* x_scales, const int* recv_src_map,
+                          int num_rows, int num_tokens, int row_bytes, int num_scales,
+                          void* recv_x, float* recv_scales, void* stream) {
+  if (num_rows < 0 || num_tokens < 0 || row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0)
+    return MI_EP_EINVAL;
+  if (!aligned16(x) || !aligned16(recv_x)) return MI_EP_EINVAL;
+  if (num_rows > 0 && (recv_src_map == nullptr || recv_x == nullptr)) return MI_EP_EINVAL;
+  if (num_rows > 0 && num_tokens > 0 && x == nullptr) return MI_EP_EINVAL;
+  if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
+  if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
+  return status_of(launch_gather_rows(static_cast<const vec16*>(x), x_scales, recv_src_map, num_rows,
+                                      num_tokens, row_bytes / 16, num_scales, static_cast<vec16*>(recv_x),
+                                      recv_scales, as_stream(stream)));
+}
+
+int mi_ep_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_source_rank,
+                       int* pull_indices, void* stream) {
+  if (num_rows < 0 || tokens_per_source_rank <= 0) return MI_EP_EINVAL;
+  if (num_rows > 0 && (recv_src_map == nullptr || pull_indices == nullptr)) return MI_EP_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(pull_indices) & 7u) != 0) return MI_EP_EINVAL;
+  return status_of(launch_pull_indices(recv_src_map, num_rows, tokens_per_source_rank, pull_indices,
+                                       as_stream(stream)));
+}
+
 int mi_ep_combine(const void* y, const int* slot_map, const float* topk_weights,
                   const void* bias_0, const void* bias_1, const float* recv_topk_weights,
                   int num_tokens, int num_topk, int hidden, void* combined_x,

@@ -115,6 +115,59 @@ __global__ __launch_bounds__(kPermuteThreads) void ep_pad_rows_kernel(const Perm
   }
 }
 
+// Pull-mode dispatch: one wave per (destination row, batch).  Destination rows are
+// written in order (a linear stream); every source row is read once per route, which
+// the caches absorb only in part -- the push kernel above is the fast path, this one
+// serves callers that hold nothing but a source map.
+template <int kBatchVecs>
+__global__ __launch_bounds__(kPermuteThreads) void ep_gather_rows_kernel(
+    const vec16* __restrict__ x, const float* __restrict__ x_scales, const int* __restrict__ recv_src_map,
+    const int num_rows, const int num_tokens, const int row_vecs, const int num_scales,
+    vec16* __restrict__ recv_x, float* __restrict__ recv_scales, const int batches_per_row) {
+  const int lane = lane_id();
+  const int wave = static_cast<int>(threadIdx.x) >> 6;
+  const long long unit = static_cast<long long>(blockIdx.x) * kPermuteWaves + wave;
+  const int row = static_cast<int>(unit / batches_per_row);
+  const int batch = static_cast<int>(unit - static_cast<long long>(row) * batches_per_row);
+  if (row >= num_rows) return;
+  const int token = recv_src_map[row];
+  const bool live = token >= 0 && token < num_tokens;
+  const vec16* src = x + static_cast<size_t>(live ? token : 0) * row_vecs;
+  vec16* dst = recv_x + static_cast<size_t>(row) * row_vecs;
+  const int v0 = batch * (kBatchVecs * kWave) + lane;
+  const vec16 zero = {0u, 0u, 0u, 0u};
+  vec16 buf[kBatchVecs];
+#pragma unroll
+  for (int u = 0; u < kBatchVecs; ++u) {
+    const int v = v0 + u * kWave;
+    buf[u] = (live && v < row_vecs) ? src[v] : zero;
+  }
+#pragma unroll
+  for (int u = 0; u < kBatchVecs; ++u) {
+    const int v = v0 + u * kWave;
+    if (v < row_vecs) __builtin_nontemporal_store(buf[u], dst + v);
+  }
+  if (batch == 0 && recv_scales != nullptr)
+    for (int j = lane; j < num_scales; j += kWave)
+      recv_scales[static_cast<size_t>(row) * num_scales + j] =
+          live ? x_scales[static_cast<size_t>(token) * num_scales + j] : 0.0f;
+}
+
+__global__ __launch_bounds__(256) void ep_pull_indices_kernel(const int* __restrict__ recv_src_map,
+                                                             const int num_rows,
+                                                             const int tokens_per_source_rank,
+                                                             int2* __restrict__ pull_indices) {
+  const int row = static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
+  if (row >= num_rows) return;
+  const int token = recv_src_map[row];
+  int2 out = {-1, -1};
+  if (token >= 0) {
+    out.x = token / tokens_per_source_rank;
+    out.y = token - out.x * tokens_per_source_rank;
+  }
+  pull_indices[row] = out;
+}
+
 __global__ __launch_bounds__(256) void ep_copy_yardstick_kernel(vec16* __restrict__ dst,
                                                                const vec16* __restrict__ src,
                                                                size_t vecs) {
@@ -156,6 +209,35 @@ hipError_t launch_permute(const PermuteArgs& a, hipStream_t stream) {
   // that a wave keeps 2 KiB of loads in flight.
   if (a.row_vecs <= kWave) return launch_permute_batch<1>(a, stream);
   return launch_permute_batch<2>(a, stream);
+}
+
+hipError_t launch_gather_rows(const vec16* x, const float* x_scales, const int* recv_src_map, int num_rows,
+                              int num_tokens, int row_vecs, int num_scales, vec16* recv_x,
+                              float* recv_scales, hipStream_t stream) {
+  if (num_rows == 0) return hipSuccess;
+  const int batch_vecs = row_vecs > kWave ? 2 : 1;
+  const int per_batch = batch_vecs * kWave;
+  const int batches = (row_vecs + per_batch - 1) / per_batch;
+  const long long units = static_cast<long long>(num_rows) * batches;
+  const long long blocks = (units + kPermuteWaves - 1) / kPermuteWaves;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  if (batch_vecs == 2)
+    hipLaunchKernelGGL((ep_gather_rows_kernel<2>), dim3(static_cast<unsigned>(blocks)), dim3(kPermuteThreads), 0,
+                       stream, x, x_scales, recv_src_map, num_rows, num_tokens, row_vecs, num_scales, recv_x,
+                       recv_scales, batches);
+  else
+    hipLaunchKernelGGL((ep_gather_rows_kernel<1>), dim3(static_cast<unsigned>(blocks)), dim3(kPermuteThreads), 0,
+                       stream, x, x_scales, recv_src_map, num_rows, num_tokens, row_vecs, num_scales, recv_x,
+                       recv_scales, batches);
+  return hipGetLastError();
+}
+
+hipError_t launch_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_source_rank,
+                               int* pull_indices, hipStream_t stream) {
+  if (num_rows == 0) return hipSuccess;
+  hipLaunchKernelGGL(ep_pull_indices_kernel, dim3((num_rows + 255) / 256), dim3(256), 0, stream, recv_src_map,
+                     num_rows, tokens_per_source_rank, reinterpret_cast<int2*>(pull_indices));
+  return hipGetLastError();
 }
 
 hipError_t launch_pad_rows(const PermuteArgs& a, hipStream_t stream) {

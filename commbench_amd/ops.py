@@ -252,6 +252,47 @@ def dispatch(x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Te
     return buf.dispatch(x, scales, topk_idx, topk_weights, expert_alignment, num_channels)
 
 
+def dispatch_cached(x: torch.Tensor, scales: Optional[torch.Tensor], recv_src_map: torch.Tensor,
+                    num_rows: Optional[int] = None):
+    """Pull-mode dispatch of a new payload with the source map of an earlier dispatch (the
+    reference's cached mode).  Returns (recv_x, recv_scales); pad rows are zero."""
+    _require(x.is_cuda and x.dim() == 2 and x.is_contiguous(), "x must be a contiguous 2-D GPU tensor")
+    _require(recv_src_map.dtype == torch.int32 and recv_src_map.dim() == 1 and recv_src_map.is_contiguous(),
+             "recv_src_map must be contiguous int32 [rows]")
+    rows = recv_src_map.shape[0] if num_rows is None else num_rows
+    _require(0 <= rows <= recv_src_map.shape[0], "num_rows exceeds the map")
+    row_bytes = x.shape[1] * x.element_size()
+    _require(row_bytes % 16 == 0, "row size must be a multiple of 16 bytes")
+    num_scales = 0
+    if scales is not None:
+        _require(scales.dtype == torch.float32 and scales.dim() == 2 and scales.is_contiguous()
+                 and scales.shape[0] == x.shape[0], "scales must be contiguous float32 [num_tokens, S]")
+        num_scales = scales.shape[1]
+    recv_x = torch.empty((rows, x.shape[1]), dtype=x.dtype, device=x.device)
+    recv_scales = (torch.empty((rows, num_scales), dtype=torch.float32, device=x.device)
+                   if scales is not None else None)
+    lib = _lib.load()
+    _lib.check(lib.mi_ep_dispatch_cached(_ptr(x), _ptr(scales), _ptr(recv_src_map), rows, x.shape[0],
+                                         row_bytes, num_scales, _ptr(recv_x), _ptr(recv_scales),
+                                         _stream()), "mi_ep_dispatch_cached")
+    return recv_x, recv_scales
+
+
+def pull_indices(recv_src_map: torch.Tensor, tokens_per_source_rank: int,
+                 num_rows: Optional[int] = None) -> torch.Tensor:
+    """The source map as {source rank, token inside the rank} pairs, {-1, -1} for pads: the
+    pull_dispatch_indices layout of the reference's ThunderKittens MoE example."""
+    _require(recv_src_map.is_cuda and recv_src_map.dtype == torch.int32 and recv_src_map.is_contiguous(),
+             "recv_src_map must be a contiguous int32 GPU tensor")
+    _require(tokens_per_source_rank > 0, "tokens_per_source_rank must be positive")
+    rows = recv_src_map.shape[0] if num_rows is None else num_rows
+    out = torch.empty((rows, 2), dtype=torch.int32, device=recv_src_map.device)
+    lib = _lib.load()
+    _lib.check(lib.mi_ep_pull_indices(_ptr(recv_src_map), rows, tokens_per_source_rank, _ptr(out),
+                                      _stream()), "mi_ep_pull_indices")
+    return out
+
+
 def copy_yardstick(dst: torch.Tensor, src: torch.Tensor) -> None:
     """16-byte streaming copy of src into dst (same byte size), the measured-bandwidth yardstick."""
     nbytes = src.numel() * src.element_size()

@@ -119,6 +119,29 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
                    float* recv_topk_weights, int* slot_map, int capacity_rows, void* stream);
 
 /*
+ * Pull-mode dispatch with a map from an earlier dispatch (the reference's cached mode,
+ * kCachedMode of dispatch_copy_epilogue_impl,
+ * example081_deepep_jit_dispatch_copy_epilogue/nv/empty_deepep_jit_dispatch_copy_epilogue.cu:11,
+ * and the token pull of the ThunderKittens MoE example,
+ * example056_thunderkitten_moe_dispatch_gemm_easy, kernel spec at :181-202): row i of
+ * recv_x / recv_scales becomes a byte copy of token recv_src_map[i]; rows whose map entry is
+ * negative (pads) or not below num_tokens are zero-filled.  No routing tables are read.
+ * Same size and alignment rules as mi_ep_dispatch.
+ */
+int mi_ep_dispatch_cached(const void* x, const float* x_scales, const int* recv_src_map,
+                          int num_rows, int num_tokens, int row_bytes, int num_scales,
+                          void* recv_x, float* recv_scales, void* stream);
+
+/*
+ * The same map in the ThunderKittens example's format
+ * (example056_thunderkitten_moe_dispatch_gemm_easy compute_dispatch_indices, :521-564):
+ * pull_indices[i] = {source rank, token index inside that rank} with tokens_per_source_rank
+ * consecutive tokens per source rank, {-1, -1} for pad rows.  int32[num_rows, 2].
+ */
+int mi_ep_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_source_rank,
+                       int* pull_indices, void* stream);
+
+/*
  * Combine: combine_impl + combine_reduce_epilogue_impl
  * (example082_deepep_jit_combine/nv/empty_deepep_jit_combine.cu:28-67,
  *  example083_deepep_jit_combine_reduce_epilogue/nv/empty_deepep_jit_combine_reduce_epilogue.cu:23-53).

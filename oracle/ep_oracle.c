@@ -23,6 +23,10 @@
  *   ep_oracle_permute           example081_deepep_jit_dispatch_copy_epilogue/nv/
  *                               empty_deepep_jit_dispatch_copy_epilogue.cu:22-60
  *                               (payload, scales, weights and source metadata per row)
+ *   ep_oracle_gather_rows,
+ *   ep_oracle_pull_indices      example056_thunderkitten_moe_dispatch_gemm_easy/nv/
+ *                               empty_thunderkitten_moe_dispatch_gemm.cu:181-202,521-564
+ *                               and the cached mode of the copy epilogue (example081 .cu:11)
  *   ep_oracle_combine           example083_deepep_jit_combine_reduce_epilogue/nv/
  *                               empty_deepep_jit_combine_reduce_epilogue.cu:23-53
  *                               (fp32 accumulate over up to K rows, two biases, bf16 out)
@@ -36,6 +40,7 @@
  *   channel prefix   closed form for the reference's routeDst pattern
  *   rank prefix      numpy cumsum over axis 0
  *   permute          numpy fancy-index gather
+ *   pull indices     the closed form of the ThunderKittens example's own generator
  *   combine          exact rational arithmetic rounded once per fma (python ints),
  *                    integer-valued exact sums, K=1 copy, closed forms
  *   bf16 codec       exhaustive against torch.bfloat16 (fixtures in tests/golden)
@@ -237,6 +242,43 @@ int ep_oracle_permute(const void* x, int row_bytes, const float* x_scales, int n
     if (recv_topk_weights) recv_topk_weights[row] = topk_weights[i];
   }
   return 0;
+}
+
+/*
+ * Pull-mode (cached) dispatch: row i is a byte copy of token src_map[i]; rows whose entry is
+ * negative or not below num_tokens are zero (example081 .cu:11 kCachedMode; example056
+ * thunderkitten_moe_dispatch_gemm_easy kernel spec :181-202).
+ */
+int ep_oracle_gather_rows(const void* x, int row_bytes, const float* x_scales, int num_scales,
+                          const int* src_map, int num_rows, int num_tokens, void* recv_x,
+                          float* recv_scales) {
+  const uint8_t* xin = (const uint8_t*)x;
+  uint8_t* xout = (uint8_t*)recv_x;
+  for (int row = 0; row < num_rows; ++row) {
+    int t = src_map[row];
+    if (t < 0 || t >= num_tokens) {
+      memset(xout + (size_t)row * row_bytes, 0, (size_t)row_bytes);
+      if (recv_scales) memset(recv_scales + (size_t)row * num_scales, 0, sizeof(float) * (size_t)num_scales);
+      continue;
+    }
+    memcpy(xout + (size_t)row * row_bytes, xin + (size_t)t * row_bytes, (size_t)row_bytes);
+    if (recv_scales)
+      memcpy(recv_scales + (size_t)row * num_scales, x_scales + (size_t)t * num_scales,
+             sizeof(float) * (size_t)num_scales);
+  }
+  return 0;
+}
+
+/*
+ * {source rank, token inside the rank} per row, {-1,-1} for pads
+ * (example056 compute_dispatch_indices, :521-564).
+ */
+void ep_oracle_pull_indices(const int* src_map, int num_rows, int tokens_per_source_rank, int* out) {
+  for (int row = 0; row < num_rows; ++row) {
+    int t = src_map[row];
+    out[2 * row] = t < 0 ? -1 : t / tokens_per_source_rank;
+    out[2 * row + 1] = t < 0 ? -1 : t % tokens_per_source_rank;
+  }
 }
 
 /* ---- combine ---------------------------------------------------------- */

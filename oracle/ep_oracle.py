@@ -143,6 +143,29 @@ def permute(x_bytes: np.ndarray, scales, topk_idx, topk_weights, src_map, src_k,
     return recv_x, recv_scales, recv_idx, recv_w
 
 
+def gather_rows(x_bytes: np.ndarray, scales, src_map: np.ndarray):
+    x_bytes = _c(x_bytes, np.uint8)
+    src_map = _c(src_map, np.int32)
+    T, row_bytes = x_bytes.shape
+    rows = src_map.shape[0]
+    recv_x = np.empty((rows, row_bytes), dtype=np.uint8)
+    num_scales, recv_scales = 0, None
+    if scales is not None:
+        scales = _c(scales, np.float32)
+        num_scales = scales.shape[1]
+        recv_scales = np.empty((rows, num_scales), dtype=np.float32)
+    _load().ep_oracle_gather_rows(_p(x_bytes), row_bytes, _p(scales), num_scales, _p(src_map), rows, T,
+                                  _p(recv_x), _p(recv_scales))
+    return recv_x, recv_scales
+
+
+def pull_indices(src_map: np.ndarray, tokens_per_source_rank: int) -> np.ndarray:
+    src_map = _c(src_map, np.int32)
+    out = np.empty((src_map.shape[0], 2), dtype=np.int32)
+    _load().ep_oracle_pull_indices(_p(src_map), src_map.shape[0], tokens_per_source_rank, _p(out))
+    return out
+
+
 def combine(y_bits: np.ndarray, slot_map: np.ndarray, topk_weights=None, bias_0=None, bias_1=None,
             num_threads: int = 1) -> np.ndarray:
     """y_bits: uint16[rows, H] bf16 bit patterns.  Returns uint16[T, H]."""

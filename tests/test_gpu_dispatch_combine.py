@@ -242,3 +242,49 @@ def test_full_size_properties_without_the_checker():
     assert torch.equal(torch.bincount(seg, minlength=E).to(torch.int32), h.num_tokens_per_expert)
     out = ops.combine(recv_x, h, w)
     assert torch.equal(out.view(torch.int16), x.view(torch.int16))
+
+
+@pytest.mark.parametrize("payload", ["bf16", "fp8"])
+def test_cached_pull_dispatch_and_pull_indices(oracle, payload):
+    """Pull-mode dispatch with the map of an earlier dispatch must reproduce that dispatch
+    (fresh payload, same routing), pads zero; pull indices in the ThunderKittens example's format."""
+    rng = np.random.default_rng(31)
+    T, K, E, R, H, align = 1500, 8, 64, 8, 2048, 128
+    topk_np = wl.zipf_distinct_topk(rng, T, E, K, 1.2)
+    topk_np[rng.random((T, K)) < 0.05] = -1
+    x_cpu = wl.bf16_normal(rng, T, H)
+    scales_cpu = None
+    if payload == "fp8":
+        x_cpu, scales_cpu = wl.quantize_fp8_blockwise(x_cpu)
+    recv_x, h, ref = dispatch_and_check(oracle, (E, R), topk_np, None, x_cpu, scales_cpu, align=align)
+    rows = int(ref["expert_offsets"][-1])
+    x2 = wl.bf16_normal(rng, T, H)
+    s2 = None
+    if payload == "fp8":
+        x2, s2 = wl.quantize_fp8_blockwise(x2)
+    got_x, got_s = ops.dispatch_cached(x2.to(gu.DEV), None if s2 is None else s2.to(gu.DEV),
+                                       h.recv_src_map, num_rows=rows)
+    want_x, want_s = oracle.gather_rows(gu.as_bytes(x2), None if s2 is None else s2.numpy(), ref["recv_src_map"])
+    np.testing.assert_array_equal(gu.as_bytes(got_x), want_x)
+    if s2 is not None:
+        np.testing.assert_array_equal(got_s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+    # and with the first payload it is the first dispatch again
+    again, _ = ops.dispatch_cached(x_cpu.to(gu.DEV), None if scales_cpu is None else scales_cpu.to(gu.DEV),
+                                   h.recv_src_map, num_rows=rows)
+    np.testing.assert_array_equal(gu.as_bytes(again), ref["recv_x"])
+    pulls = ops.pull_indices(h.recv_src_map, T // 4, num_rows=rows)
+    np.testing.assert_array_equal(pulls.cpu().numpy(), oracle.pull_indices(ref["recv_src_map"], T // 4))
+
+
+def test_rank_prefix_matrix_from_channel_prefix(oracle):
+    """One channel per source chunk: channel_prefix_matrix[dst, src] is the notify example's
+    rank_prefix_matrix[src, dst] (example047 .cu:352-360) for R contiguous source chunks."""
+    rng = np.random.default_rng(5)
+    T, K, E, R = 4096, 4, 32, 8
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    h = buf.dispatch_layout(torch.from_numpy(topk_np).to(gu.DEV), num_channels=R)
+    torch.cuda.synchronize()
+    _, _, flags = oracle.layout(topk_np, R, E)
+    counts = flags.reshape(R, T // R, R).sum(axis=1).astype(np.int32)
+    np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy().T, oracle.rank_prefix(counts))

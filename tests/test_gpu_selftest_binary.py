@@ -21,10 +21,7 @@ def test_selftest_binary_passes():
     assert len(rows) == 14                     # the reference's 7 benchmark cases on both surfaces
     assert {r["surface"] for r in rows} == {"get_dispatch_layout", "fused_layout"}
     assert all(r["throughput_avg"] > 0 for r in rows)
-    out_dir = os.path.join(ROOT, "gpurun_out")       # kept when the run's outputs are collected
-    if os.path.isdir(out_dir):
-        with open(os.path.join(out_dir, "selftest.json"), "w") as f:
-            f.write(proc.stdout)
+    print(proc.stdout)
 
 
 def test_selftest_binary_skips_without_a_device():
