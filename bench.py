@@ -29,6 +29,8 @@ def parse_args():
     ap.add_argument("--config", default="target")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short runs of the other configurations reported under other_configs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
 
@@ -37,7 +39,6 @@ class Workload:
     """Device buffers and raw C-ABI calls of one configuration (nothing allocates in a step)."""
 
     def __init__(self, cfg, dev):
-        import numpy as np
         import torch
         from commbench_amd import _lib, workloads as wl
 
@@ -154,8 +155,18 @@ def cpu_baseline(cfg, seconds):
 
     single = rate(1, seconds * 0.5)
     multi = rate(threads, seconds * 0.5) if threads > 1 else single
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
     return {"value": multi, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "single_thread_value": single,
+            "single_thread_value": single, "threads": threads, "host_nproc": os.cpu_count(),
+            "host_cpu_model": model,
             "sample": f"first {sample_tokens} tokens of the workload ({rows} routes): layout + "
                       f"offsets + slot maps + permute + combine, repeated for ~{seconds:.0f} s "
                       f"(half on 1 thread, half on {threads} OpenMP threads)"}
@@ -293,6 +304,31 @@ def main():
                      "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBPS,
                      "traffic": traffic},
     }
+    if not args.no_other_configs:
+        # Short runs of the other configurations, same step, for reference beside the headline.
+        del wk
+        torch.cuda.empty_cache()
+        others = {}
+        for name in ("c2", "c3", "c4", "c5", "target"):
+            if name == cfg.name:
+                continue
+            ocfg = wl.CONFIGS[name]
+            owk = Workload(ocfg, dev)
+            for _ in range(5):
+                owk.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(20):
+                owk.step()
+            torch.cuda.synchronize()
+            us = (time.perf_counter() - t0) * 1e6 / 20
+            others[name] = {"us_per_step": us, "tokens_per_s": ocfg.num_tokens / (us * 1e-6),
+                            "hbm_gbps_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9,
+                            "hbm_frac_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS,
+                            "num_routes": owk.num_routes}
+            del owk
+            torch.cuda.empty_cache()
+        result["other_configs"] = others
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
     print(json.dumps(result))
