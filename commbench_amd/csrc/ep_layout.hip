@@ -167,6 +167,22 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   }
   __syncthreads();
 
+  // ---- expert columns: wave bases, tile total, aggregate published at once ------
+  // (the status words need a few microseconds to reach the other tiles; the flag
+  // pass below runs in that shadow)
+  for (int col = tid; col < E; col += kLayoutThreads) {
+    int total = 0;
+#pragma unroll
+    for (int w = 0; w < kLayoutWaves; ++w) {
+      const int v = hist[w * E + col];
+      hist[w * E + col] = static_cast<uint16_t>(total);  // becomes the wave's base inside the tile
+      total += v;
+    }
+    col_total[col] = total;
+    publish(status + static_cast<size_t>(tile) * cols + col,
+            pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
+  }
+
   // ---- flags out, de-duplicated rank hits (one token per thread) ---------------
   if (tid < kTileTokens) {
     const int t = t0 + tid;
@@ -179,25 +195,19 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   }
   __syncthreads();
 
-  // ---- per column: tile total, wave bases, decoupled look-back ----------------
+  // ---- rank columns published, then the decoupled look-back of every column ------
   for (int col = tid; col < cols; col += kLayoutThreads) {
-    int total = 0;
+    int total;
+    uint64_t* mine = status + static_cast<size_t>(tile) * cols + col;
     if (col < E) {
-#pragma unroll
-      for (int w = 0; w < kLayoutWaves; ++w) {
-        const int v = hist[w * E + col];
-        hist[w * E + col] = static_cast<uint16_t>(total);  // becomes the wave's base inside the tile
-        total += v;
-      }
+      total = col_total[col];
     } else {
       total = rank_cnt[col - E];
+      col_total[col] = total;
+      publish(mine, pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
     }
-    uint64_t* mine = status + static_cast<size_t>(tile) * cols + col;
     int excl = 0;
-    if (tile == 0) {
-      publish(mine, pack_status(kFlagPrefix, gen, static_cast<uint32_t>(total)));
-    } else {
-      publish(mine, pack_status(kFlagAggregate, gen, static_cast<uint32_t>(total)));
+    if (tile != 0) {
       // Fold predecessors in, nearest first, a window of independent loads at a
       // time so that one memory round trip covers kLookbackWindow tiles.  "Tile -1"
       // is an empty prefix, which ends the walk at the front of the grid.
@@ -238,7 +248,6 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
       publish(mine, pack_status(kFlagPrefix, gen, static_cast<uint32_t>(excl + total)));
     }
     col_excl[col] = excl;
-    col_total[col] = total;
   }
   __syncthreads();
 

@@ -69,3 +69,22 @@ def test_python_surface_rejects_bad_arguments_like_the_reference():
         ops.Buffer(16, 9, 16, 8, device="cpu")
     with pytest.raises(ValueError, match="divisible"):
         ops.Buffer(16, 2, 10, 4, device="cpu")
+
+
+def test_header_is_plain_c_and_cxx(tmp_path):
+    """include/mi_ep.h must be consumable from C (the FFI boundary) and from C++."""
+    import subprocess
+    c_src = tmp_path / "use.c"
+    c_src.write_text('#include "mi_ep.h"\nint main(void) { return mi_ep_abi_version() == MI_EP_ABI_VERSION ? 0 : 1; }\n')
+    inc = os.path.join(ROOT, "include")
+    libdir = os.path.join(ROOT, "commbench_amd")
+    exe = tmp_path / "use_c"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", f"-I{inc}", str(c_src), "-o", str(exe),
+                    f"-L{libdir}", "-lmi_ep", f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    assert subprocess.run([str(exe)]).returncode == 0
+    cxx_src = tmp_path / "use.cc"
+    cxx_src.write_text('#include "mi_ep.h"\nint main() { return mi_ep_workspace_bytes(256, 8, 256, 8) == 256 + 264 * 8 ? 0 : 1; }\n')
+    exe2 = tmp_path / "use_cxx"
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", f"-I{inc}", str(cxx_src), "-o", str(exe2),
+                    f"-L{libdir}", "-lmi_ep", f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    assert subprocess.run([str(exe2)]).returncode == 0
