@@ -88,3 +88,35 @@ def test_graph_replays_match_eager(oracle):
         _, want_expert, _ = oracle.layout(t_np, R, E)
         np.testing.assert_array_equal(replayed[0], want_expert)
     _lib.check(lib.mi_ep_workspace_status(ws.data_ptr(), torch.cuda.current_stream().cuda_stream), "status")
+
+
+def test_two_streams_with_their_own_workspaces(oracle):
+    """Calls are stream-ordered and re-entrant: two buffers on two streams, interleaved launches."""
+    E, R, K, H = 64, 8, 8, 512
+    rng = np.random.default_rng(77)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    cases = []
+    for i, T in enumerate((2500, 3100)):
+        topk_np = wl.zipf_distinct_topk(rng, T, E, K, 1.2)
+        w_np = wl.softmax_gates(rng, T, K)
+        x_cpu = wl.bf16_normal(rng, T, H)
+        cases.append(dict(T=T, topk_np=topk_np, w_np=w_np, x_cpu=x_cpu, buf=ops.Buffer(T, K, E, R, device=gu.DEV),
+                          topk=torch.from_numpy(topk_np).to(gu.DEV), w=torch.from_numpy(w_np).to(gu.DEV),
+                          x=x_cpu.to(gu.DEV)))
+    torch.cuda.synchronize()
+    results = [None, None]
+    for rep in range(3):
+        for i, c in enumerate(cases):
+            with torch.cuda.stream(streams[i]):
+                recv_x, _, _, h = c["buf"].dispatch(c["x"], None, c["topk"], c["w"])
+                out = ops.combine(recv_x, h, c["w"])
+                results[i] = (recv_x, h, out)
+    torch.cuda.synchronize()
+    for c, (recv_x, h, out) in zip(cases, results):
+        ref = oracle.full_path(c["topk_np"], c["w_np"], gu.as_bytes(c["x_cpu"]), None, E, R)
+        rows = int(ref["expert_offsets"][-1])
+        np.testing.assert_array_equal(h.slot_map.cpu().numpy(), ref["slot_map"])
+        np.testing.assert_array_equal(gu.as_bytes(recv_x)[:rows], ref["recv_x"])
+        want = oracle.combine(ref["recv_x"].view(np.uint16), ref["slot_map"], c["w_np"], num_threads=8)
+        np.testing.assert_array_equal(gu.bf16_bits(out), want)
+        c["buf"].status()
