@@ -251,20 +251,32 @@ def main():
     dominant = max(names, key=lambda n: kernel_us[n])
     achieved = kernel_bytes[dominant] / (kernel_us[dominant] * 1e-6) / 1e9
 
-    # Measured streaming-copy ceiling next to the nominal peak (read + write of 1 GiB).
-    from commbench_amd import ops
+    # Measured ceilings next to the nominal peak: 16-byte streaming copy, read-only and
+    # write-only passes over the same 0.94-1 GiB buffers.
+    lib, check = wk.lib, wk._lib.check
     src = wk.y.view(torch.uint8).reshape(-1)[: 1 << 30]
     dst = wk.recv_x.view(torch.uint8).reshape(-1)[: src.numel()]
     src = src[: dst.numel()]
-    for _ in range(3):
-        ops.copy_yardstick(dst, src)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(10):
-        ops.copy_yardstick(dst, src)
-    e1.record()
-    torch.cuda.synchronize()
-    copy_gbps = 2 * src.numel() * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    nbytes = src.numel() - src.numel() % 16
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def timed(fn, moved_bytes, iters=10):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return moved_bytes * iters / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+    copy_gbps = timed(lambda: check(lib.mi_ep_copy_yardstick(dst.data_ptr(), src.data_ptr(), nbytes, wk.stream),
+                                    "copy yardstick"), 2 * nbytes)
+    read_gbps = timed(lambda: check(lib.mi_ep_read_yardstick(src.data_ptr(), nbytes, sink.data_ptr(), wk.stream),
+                                    "read yardstick"), nbytes)
+    write_gbps = timed(lambda: check(lib.mi_ep_write_yardstick(dst.data_ptr(), nbytes, wk.stream),
+                                     "write yardstick"), nbytes)
 
     traffic = None
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
@@ -300,6 +312,8 @@ def main():
         "kernel_us": kernel_us,
         "kernel_gbps": {n: kernel_bytes[n] / (kernel_us[n] * 1e-6) / 1e9 for n in names},
         "copy_yardstick_gbps": copy_gbps,
+        "read_yardstick_gbps": read_gbps,
+        "write_yardstick_gbps": write_gbps,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBPS,
                      "traffic": traffic},

@@ -253,4 +253,17 @@ int mi_ep_copy_yardstick(void* dst, const void* src, size_t bytes, void* stream)
                                          bytes / 16, as_stream(stream)));
 }
 
+int mi_ep_read_yardstick(const void* src, size_t bytes, void* sink, void* stream) {
+  if (bytes % 16 != 0 || !aligned16(src) || sink == nullptr) return MI_EP_EINVAL;
+  if (bytes > 0 && src == nullptr) return MI_EP_EINVAL;
+  return status_of(launch_read_yardstick(static_cast<const vec16*>(src), bytes / 16,
+                                         static_cast<uint32_t*>(sink), as_stream(stream)));
+}
+
+int mi_ep_write_yardstick(void* dst, size_t bytes, void* stream) {
+  if (bytes % 16 != 0 || !aligned16(dst)) return MI_EP_EINVAL;
+  if (bytes > 0 && dst == nullptr) return MI_EP_EINVAL;
+  return status_of(launch_write_yardstick(static_cast<vec16*>(dst), bytes / 16, as_stream(stream)));
+}
+
 }  // extern "C"

@@ -111,6 +111,8 @@ struct CombineArgs {
 hipError_t launch_combine(const CombineArgs& a, hipStream_t stream);
 
 hipError_t launch_copy_yardstick(vec16* dst, const vec16* src, size_t vecs, hipStream_t stream);
+hipError_t launch_read_yardstick(const vec16* src, size_t vecs, uint32_t* sink, hipStream_t stream);
+hipError_t launch_write_yardstick(vec16* dst, size_t vecs, hipStream_t stream);
 
 // ---- device helpers -------------------------------------------------------
 #ifdef __HIPCC__

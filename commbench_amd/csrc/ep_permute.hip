@@ -189,6 +189,32 @@ __global__ __launch_bounds__(256) void ep_copy_yardstick_kernel(vec16* __restric
   }
 }
 
+// Read-only stream: one pass, 4 KiB per workgroup, nothing written (the fold below can
+// only equal the magic value by accident of the data, and the store exists so that the
+// loads are not dead code).
+__global__ __launch_bounds__(256) void ep_read_yardstick_kernel(const vec16* __restrict__ src, size_t vecs,
+                                                               uint32_t* sink) {
+  constexpr int kPerThread = 4;
+  const size_t base = static_cast<size_t>(blockIdx.x) * 256 * kPerThread;
+  vec16 buf[kPerThread];
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) {
+    const size_t v = base + static_cast<size_t>(u) * 256 + threadIdx.x;
+    buf[u] = v < vecs ? __builtin_nontemporal_load(src + v) : vec16{0u, 0u, 0u, 0u};
+  }
+  uint32_t fold = 0;
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) fold ^= buf[u][0] ^ buf[u][1] ^ buf[u][2] ^ buf[u][3];
+  if (fold == 0x9e3779b9u) *sink = fold;
+}
+
+// Write-only stream: a fill, 4 KiB per workgroup.
+__global__ __launch_bounds__(256) void ep_write_yardstick_kernel(vec16* __restrict__ dst, size_t vecs) {
+  const size_t v = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const vec16 value = {0x01010101u, 0x02020202u, 0x03030303u, 0x04040404u};
+  if (v < vecs) dst[v] = value;
+}
+
 template <int kBatchVecs>
 hipError_t launch_permute_batch(const PermuteArgs& a, hipStream_t stream) {
   const int per_batch = kBatchVecs * kWave;
@@ -251,6 +277,24 @@ hipError_t launch_copy_yardstick(vec16* dst, const vec16* src, size_t vecs, hipS
   if (blocks > 8192) blocks = 8192;
   hipLaunchKernelGGL(ep_copy_yardstick_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
                      dst, src, vecs);
+  return hipGetLastError();
+}
+
+hipError_t launch_read_yardstick(const vec16* src, size_t vecs, uint32_t* sink, hipStream_t stream) {
+  if (vecs == 0) return hipSuccess;
+  const size_t blocks = (vecs + 1023) / 1024;
+  if (blocks > 0x7fffffffULL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(ep_read_yardstick_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, src,
+                     vecs, sink);
+  return hipGetLastError();
+}
+
+hipError_t launch_write_yardstick(vec16* dst, size_t vecs, hipStream_t stream) {
+  if (vecs == 0) return hipSuccess;
+  const size_t blocks = (vecs + 255) / 256;
+  if (blocks > 0x7fffffffULL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(ep_write_yardstick_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst,
+                     vecs);
   return hipGetLastError();
 }
 

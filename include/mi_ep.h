@@ -166,6 +166,13 @@ int mi_ep_combine(const void* y, const int* slot_map, const float* topk_weights,
  * bytes % 16 == 0.
  */
 int mi_ep_copy_yardstick(void* dst, const void* src, size_t bytes, void* stream);
+/* The same stream split in two: read-only (every 16-byte vector is loaded and folded into one
+ * word; *sink is written only if that word equals a fixed magic value, which keeps the loads
+ * alive without adding write traffic) and write-only (a fill).  They bound what a read-heavy
+ * (combine) and a write-heavy (permute) kernel can reach.  bytes % 16 == 0; sink is 4 bytes of
+ * device memory. */
+int mi_ep_read_yardstick(const void* src, size_t bytes, void* sink, void* stream);
+int mi_ep_write_yardstick(void* dst, size_t bytes, void* stream);
 
 #ifdef __cplusplus
 }
