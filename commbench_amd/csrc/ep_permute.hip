@@ -1,7 +1,7 @@
 // Permute (dispatch payload) kernels for gfx950.
 //
 // ep_permute_kernel: each wavefront owns (token, batch): one batch is up to
-// kBatchVecs * 64 consecutive 16-byte vectors of the token's row.  The wave reads
+// kBatchVecs * 64 consecutive 16-byte vectors of the token's row (1 KiB as launched).  The wave reads
 // its batch once into registers and stores it to every row the token was routed
 // to, so the source is read once and every destination row is written once.
 // Every access of a wave is 1 KiB contiguous.  The first batch of a token also
@@ -15,15 +15,20 @@
 namespace mi_ep {
 namespace {
 
-constexpr int kPermuteThreads = 256;
+constexpr int kPermuteThreads = 256;  // pad-row and pull-mode kernels
 constexpr int kPermuteWaves = kPermuteThreads / kWave;
+// The push kernel: small workgroups of two waves and one vector per lane measured best on
+// every row size tried (7, 8 and 14 KiB rows); the kernel is bound by HBM writes, not by
+// occupancy, and finer units even out the tail.
+constexpr int kPushThreads = 128;
+constexpr int kPushWaves = kPushThreads / kWave;
 
 template <int kBatchVecs, bool kStreamStores>
-__global__ __launch_bounds__(kPermuteThreads) void ep_permute_kernel(const PermuteArgs a,
-                                                                     const int batches_per_row) {
+__global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteArgs a,
+                                                                  const int batches_per_row) {
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
-  const long long unit = static_cast<long long>(blockIdx.x) * kPermuteWaves + wave;
+  const long long unit = static_cast<long long>(blockIdx.x) * kPushWaves + wave;
   const int token = static_cast<int>(unit / batches_per_row);
   const int batch = static_cast<int>(unit - static_cast<long long>(token) * batches_per_row);
   if (token >= a.num_tokens) return;
@@ -215,26 +220,17 @@ __global__ __launch_bounds__(256) void ep_write_yardstick_kernel(vec16* __restri
   if (v < vecs) dst[v] = value;
 }
 
-template <int kBatchVecs>
-hipError_t launch_permute_batch(const PermuteArgs& a, hipStream_t stream) {
-  const int per_batch = kBatchVecs * kWave;
-  const int batches = (a.row_vecs + per_batch - 1) / per_batch;
-  const long long units = static_cast<long long>(a.num_tokens) * batches;
-  const long long blocks = (units + kPermuteWaves - 1) / kPermuteWaves;
-  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((ep_permute_kernel<kBatchVecs, true>), dim3(static_cast<unsigned>(blocks)),
-                     dim3(kPermuteThreads), 0, stream, a, batches);
-  return hipGetLastError();
-}
-
 }  // namespace
 
 hipError_t launch_permute(const PermuteArgs& a, hipStream_t stream) {
   if (a.num_tokens == 0) return hipSuccess;
-  // Short rows fit one single-vector batch; long rows use two vectors per lane so
-  // that a wave keeps 2 KiB of loads in flight.
-  if (a.row_vecs <= kWave) return launch_permute_batch<1>(a, stream);
-  return launch_permute_batch<2>(a, stream);
+  const int batches = (a.row_vecs + kWave - 1) / kWave;
+  const long long units = static_cast<long long>(a.num_tokens) * batches;
+  const long long blocks = (units + kPushWaves - 1) / kPushWaves;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((ep_permute_kernel<1, true>), dim3(static_cast<unsigned>(blocks)), dim3(kPushThreads), 0,
+                     stream, a, batches);
+  return hipGetLastError();
 }
 
 hipError_t launch_gather_rows(const vec16* x, const float* x_scales, const int* recv_src_map, int num_rows,
