@@ -18,6 +18,7 @@ SIGNATURES = {
     "mi_ep_workspace_bytes": (_size, [_int, _int, _int, _int]),
     "mi_ep_workspace_init": (_int, [_vp, _size, _vp]),
     "mi_ep_workspace_status": (_int, [_vp, _vp]),
+    "mi_ep_set_wait_limit": (_int, [ctypes.c_uint]),
     "mi_ep_dispatch_layout": (_int, [_vp, _int, _int, _int, _int, _int, _int,
                                      _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _size, _vp]),
     "mi_ep_dispatch": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int,

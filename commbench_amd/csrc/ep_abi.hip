@@ -1,7 +1,10 @@
 // extern "C" boundary of the gfx950 dispatch core: argument checks on the host,
 // then kernel launches.  No allocation, no synchronisation (except
-// mi_ep_workspace_status, which says so), no process-wide state.
+// mi_ep_workspace_status, which says so), no process-wide state apart from the
+// wait limit of the test hook.
 #include "../../include/mi_ep.h"
+
+#include <atomic>
 
 #include "ep_device.h"
 
@@ -32,6 +35,7 @@ inline int status_of(hipError_t e) { return e == hipSuccess ? MI_EP_OK : static_
 // Bounded device-side wait: polls spaced by s_sleep, roughly a microsecond apart,
 // so a few seconds before a launch gives up and flags the workspace.
 constexpr uint32_t kSpinLimit = 1u << 22;
+std::atomic<uint32_t> g_spin_limit{kSpinLimit};  // only ever changed by the test hook
 
 }  // namespace
 
@@ -86,6 +90,11 @@ int mi_ep_workspace_status(const void* workspace, void* stream) {
   e = hipStreamSynchronize(as_stream(stream));
   if (e != hipSuccess) return static_cast<int>(e);
   return header.timed_out != 0 ? MI_EP_ETIMEDOUT : MI_EP_OK;
+}
+
+int mi_ep_set_wait_limit(unsigned int max_polls) {
+  g_spin_limit.store(max_polls == 0 ? kSpinLimit : max_polls, std::memory_order_relaxed);
+  return MI_EP_OK;
 }
 
 int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
@@ -147,7 +156,7 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
   while ((1 << a.expert_bits) < num_experts) ++a.expert_bits;
   a.inv_topk = ((1u << 19) + num_topk - 1) / num_topk;
   a.inv_experts_per_rank = ((1u << 22) + a.experts_per_rank - 1) / a.experts_per_rank;
-  a.spin_limit = kSpinLimit;
+  a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
   return status_of(launch_layout_fused(a, s));
 }
 

@@ -238,7 +238,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
           }
         }
         if (stalled) {
-          if (++spins > a.spin_limit) {
+          if (++spins >= a.spin_limit) {
             __hip_atomic_store(&a.ws->timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             break;
           }

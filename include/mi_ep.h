@@ -66,6 +66,15 @@ int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
  * workspace gave up a bounded device-side wait since the last init. */
 int mi_ep_workspace_status(const void* workspace, void* stream);
 
+/* Test hook, process-wide: bounds the number of unsuccessful polls of one device-side wait in
+ * later mi_ep_dispatch_layout launches: a wait gives up at its max_polls-th unsuccessful poll in
+ * a row (0 restores the default of about four million).  A launch
+ * whose wait expires still terminates; its outputs are then unspecified and the workspace
+ * reports MI_EP_ETIMEDOUT until it is initialised again.  The reference's counterpart is the
+ * kNumTimeoutCycles template argument of dispatch_impl
+ * (example080_deepep_jit_dispatch_payload/nv/empty_deepep_jit_dispatch_payload.cu:29,122-143). */
+int mi_ep_set_wait_limit(unsigned int max_polls);
+
 /*
  * Fused single-pass layout: everything the reference spreads over
  *   example042 (counts + flags, empty_deepep_dispatch_layout.cu:48-86),

@@ -84,6 +84,20 @@ def test_fused_layout_ragged_shapes(oracle, shape):
     gu.check_layout_against_oracle(oracle, h, topk_np, R, E, 3, 5)
 
 
+@pytest.mark.parametrize("shape", [(300000, 2, 8, 64), (131072, 8, 8, 256)], ids=lambda s: "x".join(map(str, s)))
+def test_fused_layout_more_tiles_than_resident_workgroups(oracle, shape):
+    """Over a thousand tiles: more workgroups than the device holds at once.  Tiles are handed out
+    by ticket, so a tile only ever waits on tiles that have already started."""
+    T, K, R, E = shape
+    print(f"shape {shape}", flush=True)
+    rng = np.random.default_rng(T)
+    topk_np = wl.zipf_distinct_topk(rng, T, E, K, 1.2) if K == 8 else rng.integers(-1, E, size=(T, K)).astype(np.int64)
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    for _ in range(2):
+        _, h = gu.run_fused_layout(buf, topk_np, expert_alignment=16, num_channels=16)
+    gu.check_layout_against_oracle(oracle, h, topk_np, R, E, 16, 16)
+
+
 def test_fused_layout_out_of_range_and_all_masked(oracle):
     T, K, R, E = 700, 4, 4, 16
     rng = np.random.default_rng(5)
@@ -130,3 +144,35 @@ def test_channel_prefix_reference_notify_cases(oracle, T, R):
     _, h = gu.run_fused_layout(buf, topk_np, num_channels=C)
     np.testing.assert_array_equal(h.is_token_in_rank.cpu().numpy().view(np.uint8), flags)
     np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy(), oracle.channel_prefix(flags, C))
+
+
+def test_expired_wait_terminates_and_is_reported(oracle):
+    """Failure handling without a hang: with the wait limit forced to one poll, a launch over many
+    tiles gives up at least one look-back wait; it must still finish, the workspace must report
+    it, and after re-initialisation the same workspace must work again."""
+    from commbench_amd import _lib
+    lib = _lib.load()
+    T, K, R, E = 65536, 8, 8, 256
+    topk_np = wl.uniform_distinct_topk(np.random.default_rng(3), T, E, K)
+    topk = torch.from_numpy(topk_np).to(gu.DEV)
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    try:
+        assert lib.mi_ep_set_wait_limit(1) == 0
+        expired = False
+        for _ in range(20):                       # every launch terminates; some wait will expire
+            buf.dispatch_layout(topk)
+            torch.cuda.synchronize()
+            code = lib.mi_ep_workspace_status(buf.workspace.data_ptr(), torch.cuda.current_stream().cuda_stream)
+            if code != 0:
+                assert code == -110 and _lib.strerror(code) == "device-side wait timed out"
+                expired = True
+                break
+        assert expired, "no wait expired with a one-poll limit over 256 tiles"
+        with pytest.raises(_lib.MiEpError):
+            buf.status()
+    finally:
+        assert lib.mi_ep_set_wait_limit(0) == 0
+    _lib.check(lib.mi_ep_workspace_init(buf.workspace.data_ptr(), buf.workspace.numel(),
+                                        torch.cuda.current_stream().cuda_stream), "re-init")
+    _, h = gu.run_fused_layout(buf, topk_np)
+    gu.check_layout_against_oracle(oracle, h, topk_np, R, E)
