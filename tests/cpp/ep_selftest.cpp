@@ -112,7 +112,6 @@ bool check_counts_surface(const Case& c) {
   layout.compute(d_idx.p, d_rank.p, d_expert.p, d_flags.p);  // relaunch without re-zeroing (:313-329)
   MI_EP_HIP_CHECK(hipDeviceSynchronize());
   bool ok = d_rank.download(c.ranks) == ref.per_rank && d_expert.download(c.experts) == ref.per_expert;
-  const std::vector<bool> dummy;
   std::vector<uint8_t> got(ref.flags.size());
   MI_EP_HIP_CHECK(hipMemcpy(got.data(), d_flags.p, got.size(), hipMemcpyDeviceToHost));
   for (size_t i = 0; i < got.size(); ++i) ok = ok && ((got[i] != 0) == (ref.flags[i] != 0));
@@ -213,6 +212,8 @@ struct MetricRow {
   std::string surface;
   Case c;
   double latency_us = 0.0, mtokens_per_s = 0.0;
+  int hidden = 0;             // payload rows only
+  double data_bytes = 0.0;    // the reference harness's own data-size formula for the row
 };
 
 template <class Launch>
@@ -250,6 +251,37 @@ void benchmark_case(const Case& c, std::vector<MetricRow>* rows) {
   buf.check_status();
 }
 
+// Dispatch (fused layout + permute) and combine at one shape, timed the same way.  data_bytes
+// follows the reference harnesses: index bytes for dispatch
+// (example080 build_and_run.py:761-765: T*K*8 + T*K*4 + workgroups*R*4, the last term taken as
+// tiles*R*4 here) and payload bytes for combine (example082 build_and_run.py:778-782:
+// n*H*2 + T*H*2 + T*K*4).
+void benchmark_payload_case(const Case& c, int hidden, std::vector<MetricRow>* rows) {
+  const std::vector<TopkIdx> idx = make_topk(c);
+  std::vector<float> w(idx.size(), 1.0f / c.topk);
+  DeviceArray<TopkIdx> d_idx(idx.size());
+  DeviceArray<float> d_w(w.size());
+  DeviceArray<uint16_t> d_x(static_cast<size_t>(c.tokens) * hidden), d_out(static_cast<size_t>(c.tokens) * hidden);
+  d_idx.upload(idx);
+  d_w.upload(w);
+  d_x.fill_bytes(0x3c);
+  mi_ep::ExpertParallelBuffer buf(c.tokens, c.topk, c.experts, c.ranks);
+  DeviceArray<uint16_t> d_recv(static_cast<size_t>(buf.capacity_rows()) * hidden);
+  d_recv.fill_bytes(0x3c);
+  const double n = static_cast<double>(c.tokens) * c.topk;  // no masked slots in these patterns
+  MetricRow d = time_launches("dispatch", c, [&] {
+    buf.dispatch(d_x.p, nullptr, d_idx.p, d_w.p, c.tokens, hidden * 2, 0, d_recv.p, nullptr);
+  });
+  d.hidden = hidden;
+  d.data_bytes = n * 8 + n * 4 + ((c.tokens + 255) / 256) * c.ranks * 4.0;
+  rows->push_back(d);
+  MetricRow m = time_launches("combine", c, [&] { buf.combine(d_recv.p, d_w.p, nullptr, nullptr, hidden, d_out.p); });
+  m.hidden = hidden;
+  m.data_bytes = n * hidden * 2 + static_cast<double>(c.tokens) * hidden * 2 + n * 4;
+  rows->push_back(m);
+  buf.check_status();
+}
+
 void print_json(bool pass, const std::vector<MetricRow>& rows) {
   std::cout << std::fixed << std::setprecision(3);
   std::cout << "{\n  \"Correctness\": \"" << (pass ? "PASS" : "FAIL") << "\",\n";
@@ -260,7 +292,11 @@ void print_json(bool pass, const std::vector<MetricRow>& rows) {
     std::cout << "    {\"surface\": \"" << r.surface << "\", \"data_size\": " << r.c.tokens << ", \"num_topk\": " << r.c.topk
               << ", \"num_ranks\": " << r.c.ranks << ", \"num_experts\": " << r.c.experts << ", \"pattern\": \""
               << pattern_name(r.c.pattern) << "\", \"throughput_avg\": " << r.mtokens_per_s
-              << ", \"latency_avg\": " << r.latency_us << "}" << (i + 1 != rows.size() ? "," : "") << "\n";
+              << ", \"latency_avg\": " << r.latency_us;
+    if (r.hidden > 0)
+      std::cout << ", \"hidden\": " << r.hidden << ", \"data_bytes\": " << r.data_bytes
+                << ", \"gbytes_per_s\": " << (r.latency_us > 0.0 ? r.data_bytes / r.latency_us / 1e3 : 0.0);
+    std::cout << "}" << (i + 1 != rows.size() ? "," : "") << "\n";
   }
   std::cout << "  ]\n}\n";
 }
@@ -310,6 +346,9 @@ int main(int argc, char** argv) {
     benchmark_case({65536, 4, 8, 32, kRankSweep}, &rows);
     benchmark_case({65536, 8, 8, 32, kSameRank}, &rows);
     benchmark_case({65536, 2, 4, 32, kSpread}, &rows);
+    // The JIT examples' default shape (example080 build_and_run.py:542-548) and the large shape.
+    benchmark_payload_case({512, 2, 8, 64, kSpread}, 256, &rows);
+    benchmark_payload_case({8192, 8, 8, 256, kSpread}, 7168, &rows);
   }
   print_json(pass, rows);
   return pass ? 0 : 1;
