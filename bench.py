@@ -110,7 +110,7 @@ class Workload:
     def combine(self):
         c = self.cfg
         self._lib.check(self.lib.mi_ep_combine(
-            self.y.data_ptr(), self.slot_map.data_ptr(), self.w.data_ptr(), None, None, None,
+            self.y.data_ptr(), self.cap, self.slot_map.data_ptr(), self.w.data_ptr(), None, None, None,
             c.num_tokens, c.num_topk, c.hidden, self.out.data_ptr(), None, self.stream), "combine")
 
     def step(self):

@@ -229,12 +229,13 @@ int mi_ep_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_sou
                                        as_stream(stream)));
 }
 
-int mi_ep_combine(const void* y, const int* slot_map, const float* topk_weights,
+int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
                   const void* bias_0, const void* bias_1, const float* recv_topk_weights,
                   int num_tokens, int num_topk, int hidden, void* combined_x,
                   float* combined_topk_weights, void* stream) {
   if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK) return MI_EP_EINVAL;
-  if (hidden <= 0 || hidden % 8 != 0) return MI_EP_EINVAL;
+  if (hidden <= 0 || hidden % 8 != 0 || num_rows < 0) return MI_EP_EINVAL;
+  if (num_rows > 0 && y == nullptr) return MI_EP_EINVAL;
   if ((recv_topk_weights != nullptr) != (combined_topk_weights != nullptr)) return MI_EP_EINVAL;
   if (num_tokens > 0 && (slot_map == nullptr || combined_x == nullptr)) return MI_EP_EINVAL;
   if (!aligned16(y) || !aligned16(bias_0) || !aligned16(bias_1) || !aligned16(combined_x))
@@ -251,6 +252,7 @@ int mi_ep_combine(const void* y, const int* slot_map, const float* topk_weights,
   a.combined_topk_weights = combined_topk_weights;
   a.num_tokens = num_tokens;
   a.num_topk = num_topk;
+  a.num_rows = num_rows;
   a.row_vecs = hidden / 8;
   return status_of(launch_combine(a, as_stream(stream)));
 }

@@ -41,6 +41,7 @@ __device__ __forceinline__ void combine_unit(const CombineArgs& a, const int tok
   if (lane < kTopk) {
     const size_t i = static_cast<size_t>(token) * kTopk + lane;
     slot = a.slot_map[i];
+    if (slot >= a.num_rows) slot = -1;
     if (a.topk_weights != nullptr) weight = a.topk_weights[i];
     if (batch == 0 && a.combined_topk_weights != nullptr)
       a.combined_topk_weights[i] = slot >= 0 ? a.recv_topk_weights[slot] : 0.0f;

@@ -105,6 +105,7 @@ struct CombineArgs {
   float* combined_topk_weights;
   int num_tokens;
   int num_topk;
+  int num_rows;  // rows of y; map entries at or beyond it are treated as non-routes
   int row_vecs;  // 16-byte vectors (8 bf16) per row
 };
 

@@ -235,7 +235,7 @@ def combine(y: torch.Tensor, slot_map: Union[torch.Tensor, DispatchHandle],
     out_w = (torch.empty((T, K), dtype=torch.float32, device=dev)
              if recv_topk_weights is not None else None)
     lib = _lib.load()
-    _lib.check(lib.mi_ep_combine(_ptr(y), _ptr(slot_map), _ptr(topk_weights), _ptr(bias_0),
+    _lib.check(lib.mi_ep_combine(_ptr(y), y.shape[0], _ptr(slot_map), _ptr(topk_weights), _ptr(bias_0),
                                  _ptr(bias_1), _ptr(recv_topk_weights), T, K, H, _ptr(out),
                                  _ptr(out_w), _stream()), "mi_ep_combine")
     if out_w is not None:

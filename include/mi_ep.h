@@ -158,13 +158,14 @@ int mi_ep_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_sou
  * accumulated in fp32, slots ascending, one fused multiply-add per row, one
  * rounding to bf16 at the end.  topk_weights == NULL gives the reference's plain
  * ordered sum.  hidden % 8 == 0; y, biases and combined_x 16-byte aligned.
- *   y            bf16[*, hidden] expert outputs in dispatch row order
+ *   y            bf16[num_rows, hidden] expert outputs in dispatch row order; map entries
+ *                that are negative or not below num_rows are not routes
  *   bias_0/1     bf16[num_tokens, hidden] or NULL
  *   recv_topk_weights / combined_topk_weights   both NULL, or float[rows] in and
  *                float[num_tokens, num_topk] out: the weights that travelled with the
  *                rows, gathered back per route (0 for non-routes)
  */
-int mi_ep_combine(const void* y, const int* slot_map, const float* topk_weights,
+int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
                   const void* bias_0, const void* bias_1, const float* recv_topk_weights,
                   int num_tokens, int num_topk, int hidden, void* combined_x,
                   float* combined_topk_weights, void* stream);

@@ -173,10 +173,11 @@ class ExpertParallelBuffer {
   }
 
   // combined_x[t] = bf16(sum_k w[t,k] * y[slot_map[t,k]] + bias_0 + bias_1); null weights = plain sum.
-  void combine(const void* d_y, const float* d_topk_weights, const void* d_bias_0, const void* d_bias_1,
-               int hidden, void* d_combined_x, float* d_combined_topk_weights = nullptr,
-               hipStream_t stream = 0) const {
-    MI_EP_CHECK(mi_ep_combine(d_y, h_.slot_map, d_topk_weights, d_bias_0, d_bias_1,
+  // d_y holds num_rows rows (capacity_rows() when it is the buffer dispatch filled).
+  void combine(const void* d_y, int num_rows, const float* d_topk_weights, const void* d_bias_0,
+               const void* d_bias_1, int hidden, void* d_combined_x,
+               float* d_combined_topk_weights = nullptr, hipStream_t stream = 0) const {
+    MI_EP_CHECK(mi_ep_combine(d_y, num_rows, h_.slot_map, d_topk_weights, d_bias_0, d_bias_1,
                               d_combined_topk_weights != nullptr ? h_.recv_topk_weights : nullptr,
                               h_.num_tokens, num_topk_, hidden, d_combined_x, d_combined_topk_weights,
                               stream));

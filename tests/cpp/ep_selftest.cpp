@@ -197,7 +197,7 @@ bool check_round_trip() {
   mi_ep::ExpertParallelBuffer buf(c.tokens, c.topk, c.experts, c.ranks);
   DeviceArray<uint16_t> d_recv(static_cast<size_t>(buf.capacity_rows()) * hidden);
   const mi_ep::DispatchHandle& h = buf.dispatch(d_x.p, nullptr, d_idx.p, d_w.p, c.tokens, row_bytes, 0, d_recv.p, nullptr);
-  buf.combine(d_recv.p, d_w.p, nullptr, nullptr, hidden, d_out.p);
+  buf.combine(d_recv.p, buf.capacity_rows(), d_w.p, nullptr, nullptr, hidden, d_out.p);
   buf.check_status();
   bool ok = d_recv.download(want_recv.size()) == want_recv;
   std::vector<int> got_map(ref.slot_map.size()), got_src(rows);
@@ -275,7 +275,7 @@ void benchmark_payload_case(const Case& c, int hidden, std::vector<MetricRow>* r
   d.hidden = hidden;
   d.data_bytes = n * 8 + n * 4 + ((c.tokens + 255) / 256) * c.ranks * 4.0;
   rows->push_back(d);
-  MetricRow m = time_launches("combine", c, [&] { buf.combine(d_recv.p, d_w.p, nullptr, nullptr, hidden, d_out.p); });
+  MetricRow m = time_launches("combine", c, [&] { buf.combine(d_recv.p, buf.capacity_rows(), d_w.p, nullptr, nullptr, hidden, d_out.p); });
   m.hidden = hidden;
   m.data_bytes = n * hidden * 2 + static_cast<double>(c.tokens) * hidden * 2 + n * 4;
   rows->push_back(m);

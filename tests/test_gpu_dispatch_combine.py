@@ -288,3 +288,21 @@ def test_rank_prefix_matrix_from_channel_prefix(oracle):
     _, _, flags = oracle.layout(topk_np, R, E)
     counts = flags.reshape(R, T // R, R).sum(axis=1).astype(np.int32)
     np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy().T, oracle.rank_prefix(counts))
+
+
+def test_combine_ignores_map_entries_beyond_the_rows_it_was_given(oracle):
+    """Memory safety: a map entry at or beyond y's row count is treated as a non-route, never read."""
+    rng = np.random.default_rng(41)
+    T, K, E, R, H = 600, 4, 16, 4, 256
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    w_np = wl.softmax_gates(rng, T, K)
+    _, per_expert, _ = oracle.layout(topk_np, R, E)
+    off, _ = oracle.expert_offsets(per_expert, R, 1)
+    _, slot_map, _, _ = oracle.slot_maps(topk_np, E, off)
+    rows_given = int(off[-1]) // 2
+    y = wl.bf16_normal(rng, rows_given, H).to(gu.DEV)
+    out = ops.combine(y, torch.from_numpy(slot_map).to(gu.DEV), torch.from_numpy(w_np).to(gu.DEV))
+    torch.cuda.synchronize()
+    clipped = np.where(slot_map < rows_given, slot_map, -1).astype(np.int32)
+    want = oracle.combine(gu.bf16_bits(y), clipped, w_np)
+    np.testing.assert_array_equal(gu.bf16_bits(out), want)
