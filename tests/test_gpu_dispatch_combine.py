@@ -306,3 +306,24 @@ def test_combine_ignores_map_entries_beyond_the_rows_it_was_given(oracle):
     clipped = np.where(slot_map < rows_given, slot_map, -1).astype(np.int32)
     want = oracle.combine(gu.bf16_bits(y), clipped, w_np)
     np.testing.assert_array_equal(gu.bf16_bits(out), want)
+
+
+@pytest.mark.parametrize("kind", ["one_expert", "two_experts_alternating", "last_expert_only"])
+def test_extreme_skew_round_trip(oracle, kind):
+    """Every route on one or two experts (with duplicates inside each token): one giant segment,
+    every lane of every wave in the same ballot group."""
+    T, K, E, R, H = 3000, 8, 64, 8, 512
+    if kind == "one_expert":
+        topk_np = np.full((T, K), 5, dtype=np.int64)
+    elif kind == "two_experts_alternating":
+        topk_np = np.tile(np.array([7, 40] * (K // 2), dtype=np.int64), (T, 1))
+    else:
+        topk_np = np.full((T, K), -1, dtype=np.int64)
+        topk_np[:, K - 1] = E - 1
+    rng = np.random.default_rng(9)
+    w_np = wl.softmax_gates(rng, T, K)
+    x_cpu = wl.bf16_normal(rng, T, H)
+    recv_x, h, ref = dispatch_and_check(oracle, (E, R), topk_np, w_np, x_cpu, None, align=128)
+    rows = int(ref["expert_offsets"][-1])
+    got, want, worst = combine_and_check(oracle, recv_x[:rows].contiguous(), h.slot_map, w_np, ref["slot_map"])
+    assert worst == 0
