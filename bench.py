@@ -245,8 +245,10 @@ def main():
     staged = T >= 16 * cus and 2048 <= cfg.hidden * 2 <= 160 * 1024
     names = ["ep_layout_fused_kernel", "ep_permute_kernel",
              "ep_combine_staged_kernel" if staged else "ep_combine_kernel"]
-    kernel_us = {n: sum(ev[i].elapsed_time(ev[i + 1]) for ev in marks) * 1e3 / args.steps
-                 for i, n in enumerate(names)}
+    per_step = {n: sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for ev in marks) for i, n in enumerate(names)}
+    kernel_us = {n: sum(v) / len(v) for n, v in per_step.items()}
+    kernel_us_stats = {n: {"avg": sum(v) / len(v), "median": v[len(v) // 2], "min": v[0]}
+                       for n, v in per_step.items()}
     kernel_bytes = dict(zip(names, (wk.bytes["layout"], wk.bytes["dispatch"], wk.bytes["combine"])))
     dominant = max(names, key=lambda n: kernel_us[n])
     achieved = kernel_bytes[dominant] / (kernel_us[dominant] * 1e-6) / 1e9
@@ -310,6 +312,7 @@ def main():
         "graph_replay_ms_per_step": graph_ms_per_step,
         "algorithmic_bytes": wk.bytes,
         "kernel_us": kernel_us,
+        "kernel_us_stats": kernel_us_stats,
         "kernel_gbps": {n: kernel_bytes[n] / (kernel_us[n] * 1e-6) / 1e9 for n in names},
         "copy_yardstick_gbps": copy_gbps,
         "read_yardstick_gbps": read_gbps,

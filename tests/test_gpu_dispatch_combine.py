@@ -327,3 +327,29 @@ def test_extreme_skew_round_trip(oracle, kind):
     rows = int(ref["expert_offsets"][-1])
     got, want, worst = combine_and_check(oracle, recv_x[:rows].contiguous(), h.slot_map, w_np, ref["slot_map"])
     assert worst == 0
+
+
+def test_combine_denormals_infinities_and_nans(oracle):
+    """Special values go through the same arithmetic on both sides: fp32 denormals are kept, an
+    infinity times a zero weight is NaN, NaNs stay NaNs (quiet bit set), signed zeros survive."""
+    rng = np.random.default_rng(23)
+    T, K, E, R, H = 400, 4, 16, 4, 64
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    _, per_expert, _ = oracle.layout(topk_np, R, E)
+    off, _ = oracle.expert_offsets(per_expert, R, 1)
+    _, slot_map, _, _ = oracle.slot_maps(topk_np, E, off)
+    rows = int(off[-1])
+    specials = np.array([0x0000, 0x8000, 0x0001, 0x8001, 0x007F, 0x0080, 0x7F7F, 0xFF7F, 0x7F80, 0xFF80,
+                         0x7FC0, 0x7F81, 0x3F80, 0xBF80], dtype=np.uint16)
+    y_bits = specials[rng.integers(0, specials.size, size=(rows, H))]
+    y = torch.from_numpy(y_bits.view(np.int16)).view(torch.bfloat16).to(gu.DEV)
+    w_np = rng.choice(np.array([0.0, -0.0, 0.5, 1.0, 2.0 ** -20, -3.0], dtype=np.float32), size=(T, K))
+    out = ops.combine(y, torch.from_numpy(slot_map).to(gu.DEV), torch.from_numpy(w_np).to(gu.DEV))
+    torch.cuda.synchronize()
+    want = oracle.combine(y_bits, slot_map, w_np)
+    got = gu.bf16_bits(out)
+    is_nan = lambda b: ((b & 0x7F80) == 0x7F80) & ((b & 0x007F) != 0)
+    np.testing.assert_array_equal(is_nan(got), is_nan(want))
+    keep = ~is_nan(want)
+    np.testing.assert_array_equal(got[keep], want[keep])
+    assert is_nan(want).any() and ((want & 0x7F80) == 0).any()      # the case really has both
