@@ -29,6 +29,9 @@ def parse_args():
     ap.add_argument("--config", default="target")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--rotate-x", type=int, default=1,
+                    help="number of distinct source buffers cycled through by consecutive steps "
+                         "(3 or more keeps the source out of the 256 MB memory-side cache)")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short runs of the other configurations reported under other_configs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -38,7 +41,7 @@ def parse_args():
 class Workload:
     """Device buffers and raw C-ABI calls of one configuration (nothing allocates in a step)."""
 
-    def __init__(self, cfg, dev):
+    def __init__(self, cfg, dev, rotate_x=1):
         import torch
         from commbench_amd import _lib, workloads as wl
 
@@ -58,6 +61,8 @@ class Workload:
             self.scales = torch.where(amax > 0, amax / 448.0, torch.ones_like(amax)).contiguous()
             x = (xf / self.scales[:, :, None]).clamp_(-448, 448).to(torch.float8_e4m3fn).view(T, H)
         self.x = x.contiguous()
+        self.x_ring = [self.x] + [self.x.clone() for _ in range(max(0, rotate_x - 1))]
+        self.step_index = 0
         cap = T * K
         self.cap = cap
         self.recv_x = torch.empty((cap, H), dtype=self.x.dtype, device=dev)
@@ -98,8 +103,10 @@ class Workload:
 
     def dispatch(self):
         c = self.cfg
+        x = self.x_ring[self.step_index % len(self.x_ring)]
+        self.step_index += 1
         self._lib.check(self.lib.mi_ep_dispatch(
-            self.x.data_ptr(), None if self.scales is None else self.scales.data_ptr(),
+            x.data_ptr(), None if self.scales is None else self.scales.data_ptr(),
             self.topk.data_ptr(), self.w.data_ptr(), self.off.data_ptr(), self.slot_rel.data_ptr(),
             self.per_expert.data_ptr(), c.num_tokens, c.num_topk, c.num_experts, 1, c.row_bytes,
             c.num_scales, self.recv_x.data_ptr(),
@@ -186,7 +193,7 @@ def main():
     cfg = wl.CONFIGS[args.config]
     dev = "cuda:0"
     torch.cuda.set_device(0)
-    wk = Workload(cfg, dev)
+    wk = Workload(cfg, dev, args.rotate_x)
     T = cfg.num_tokens
 
     for _ in range(args.warmup):
@@ -201,6 +208,24 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
+
+    # The same steps with the source rows cycling through three buffers, so that they come from
+    # HBM instead of the 256 MB memory-side cache that keeps a single re-read source resident.
+    cold_ms_per_step = None
+    if len(wk.x_ring) == 1:
+        ring = wk.x_ring
+        wk.x_ring = [wk.x, wk.x.clone(), wk.x.clone()]
+        for _ in range(6):
+            wk.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            wk.step()
+        torch.cuda.synchronize()
+        cold_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+        wk.x_ring = ring
+        wk.step()
+        torch.cuda.synchronize()
 
     # The same steps replayed as one HIP graph of the three kernels (no host launch gaps).
     graph_ms_per_step = None
@@ -306,10 +331,16 @@ def main():
                         f"{wk.num_routes} routes",
             "num_tokens": T, "hidden": cfg.hidden, "num_experts": cfg.num_experts,
             "num_topk": cfg.num_topk, "num_ranks": cfg.num_ranks, "payload": cfg.payload,
+            "source_buffers": args.rotate_x,
         },
         "hbm_gbps_whole_step": wk.bytes["total"] / (ms_per_step * 1e-3) / 1e9,
         "hbm_frac_whole_step": wk.bytes["total"] / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
         "graph_replay_ms_per_step": graph_ms_per_step,
+        "cold_source": None if cold_ms_per_step is None else {
+            "ms_per_step": cold_ms_per_step,
+            "tokens_per_s": T / (cold_ms_per_step * 1e-3),
+            "hbm_frac_whole_step": wk.bytes["total"] / (cold_ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+            "note": "source rows cycled through 3 buffers so that they are read from HBM"},
         "algorithmic_bytes": wk.bytes,
         "kernel_us": kernel_us,
         "kernel_us_stats": kernel_us_stats,
