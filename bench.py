@@ -32,6 +32,8 @@ def parse_args():
     ap.add_argument("--rotate-x", type=int, default=1,
                     help="number of distinct source buffers cycled through by consecutive steps "
                          "(3 or more keeps the source out of the 256 MB memory-side cache)")
+    ap.add_argument("--no-cold-source", action="store_true",
+                    help="skip the extra pass with the source rows cycling through three buffers")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short runs of the other configurations reported under other_configs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -212,7 +214,7 @@ def main():
     # The same steps with the source rows cycling through three buffers, so that they come from
     # HBM instead of the 256 MB memory-side cache that keeps a single re-read source resident.
     cold_ms_per_step = None
-    if len(wk.x_ring) == 1:
+    if len(wk.x_ring) == 1 and not args.no_cold_source:
         ring = wk.x_ring
         wk.x_ring = [wk.x, wk.x.clone(), wk.x.clone()]
         for _ in range(6):
