@@ -100,7 +100,7 @@ class Workload:
         self._lib.check(self.lib.mi_ep_dispatch_layout(
             self.topk.data_ptr(), c.num_tokens, c.num_topk, c.num_ranks, c.num_experts, 1, 0,
             self.per_rank.data_ptr(), self.per_expert.data_ptr(), self.in_rank.data_ptr(),
-            self.off.data_ptr(), self.psum.data_ptr(), None, self.slot_rel.data_ptr(),
+            self.off.data_ptr(), self.psum.data_ptr(), None, self.slot_rel.data_ptr(), None, 0,
             self.ws.data_ptr(), self.ws.numel(), self.stream), "layout")
 
     def dispatch(self):

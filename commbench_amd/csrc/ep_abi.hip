@@ -101,8 +101,8 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
                           int num_experts, int expert_alignment, int num_channels,
                           int* num_tokens_per_rank, int* num_tokens_per_expert,
                           bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
-                          int* channel_prefix_matrix, int* slot_rel, void* workspace,
-                          size_t workspace_bytes, void* stream) {
+                          int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
+                          int rank_slot_base, void* workspace, size_t workspace_bytes, void* stream) {
   if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
   if (expert_alignment < 1) return MI_EP_EINVAL;
   if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
@@ -143,6 +143,8 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
   a.psum_rank_rows = psum_rank_rows;
   a.channel_prefix_matrix = channel_prefix_matrix;
   a.slot_rel = slot_rel;
+  a.rank_slot_idx = rank_slot_idx;
+  a.rank_slot_base = rank_slot_base;
   a.ws = static_cast<LayoutWorkspace*>(workspace);
   a.num_tokens = num_tokens;
   a.num_topk = num_topk;

@@ -40,6 +40,7 @@ struct LayoutArgs {
   int* psum_rank_rows;
   int* channel_prefix_matrix;
   int* slot_rel;
+  int* rank_slot_idx;
   LayoutWorkspace* ws;
   int num_tokens;
   int num_topk;
@@ -49,6 +50,7 @@ struct LayoutArgs {
   int expert_alignment;
   int num_channels;
   int num_tiles;
+  int rank_slot_base;
   int expert_bits;  // ceil(log2(num_experts)), at least 1
   uint32_t inv_topk;              // ceil(2^19 / num_topk): n / num_topk == (n * inv) >> 19 for n < 2048
   uint32_t inv_experts_per_rank;  // ceil(2^22 / experts_per_rank): exact for e < 1024

@@ -85,7 +85,8 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   int* rank_cnt = col_excl + cols;          // [kMaxRanks]
   int* wave_sums = rank_cnt + kMaxRanks;    // [kLayoutWaves]
   int* misc = wave_sums + kLayoutWaves;     // [4] tile, generation
-  int* offs = misc + 4;                     // [E + 2] offsets staged by the last tile
+  int* rank_wave = misc + 4;                // [kTileTokens / kWave][kMaxRanks] flagged tokens per wave
+  int* offs = rank_wave + (kTileTokens / kWave) * kMaxRanks;  // [E + 2] offsets staged by the last tile
   uint64_t* tok_flags = reinterpret_cast<uint64_t*>(offs + E + 2 + (E & 1));  // [kTileTokens], byte r = rank r
   uint16_t* hist = reinterpret_cast<uint16_t*>(tok_flags + kTileTokens);  // [kLayoutWaves][E] wave-private
 
@@ -266,6 +267,49 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     }
   }
 
+  // ---- the deterministic prologue's table: per destination rank, tokens take slots in
+  // token order; the first slot of a token that reaches the rank carries the slot number
+  if (a.rank_slot_idx != nullptr) {
+    int below[kMaxRanks];
+    uint64_t f = 0;
+    if (tid < kTileTokens) {
+      f = tok_flags[tid];
+#pragma unroll
+      for (int r = 0; r < kMaxRanks; ++r) {
+        const uint64_t hit = __ballot(r < R && ((f >> (8 * r)) & 1u) != 0);
+        below[r] = __popcll(hit & lanes_below(lane));
+        if (lane == 0) rank_wave[wave * kMaxRanks + r] = __popcll(hit);
+      }
+    }
+    __syncthreads();
+    const int t = t0 + tid;
+    if (tid < kTileTokens && t < T) {
+      int position[kMaxRanks];
+#pragma unroll
+      for (int r = 0; r < kMaxRanks; ++r) {
+        int base = r < R ? col_excl[E + r] : 0;
+        for (int w = 0; w < wave; ++w) base += rank_wave[w * kMaxRanks + r];
+        position[r] = a.rank_slot_base + base + below[r];
+      }
+      uint32_t seen = 0;
+      for (int k = 0; k < K; ++k) {
+        const int64_t e64 = a.topk_idx[static_cast<size_t>(t) * K + k];
+        int out = -1;
+        if (e64 >= 0 && e64 < static_cast<int64_t>(E)) {
+          const int rank = static_cast<int>((static_cast<uint32_t>(e64) * a.inv_experts_per_rank) >> 22);
+          if (((seen >> rank) & 1u) == 0) {
+            seen |= 1u << rank;
+            int slot = 0;
+#pragma unroll
+            for (int r = 0; r < kMaxRanks; ++r) slot = (r == rank) ? position[r] : slot;
+            out = slot;
+          }
+        }
+        a.rank_slot_idx[static_cast<size_t>(t) * K + k] = out;
+      }
+    }
+  }
+
   // ---- per-channel inclusive prefix: the tile holding a channel's end writes it
   if (a.channel_prefix_matrix != nullptr) {
     const int C = a.num_channels;
@@ -424,7 +468,8 @@ hipError_t launch_layout_fused(const LayoutArgs& a, hipStream_t stream) {
   static_assert(kMaxExperts <= kLayoutThreads, "the offset scan takes one expert per thread");
   const int E = a.num_experts;
   const int cols = E + a.num_ranks;
-  const size_t lds = sizeof(int) * (2 * static_cast<size_t>(cols) + kMaxRanks + kLayoutWaves + 4 + E + 2 + (E & 1)) +
+  const size_t lds = sizeof(int) * (2 * static_cast<size_t>(cols) + kMaxRanks + kLayoutWaves + 4 +
+                                    (kTileTokens / kWave) * kMaxRanks + E + 2 + (E & 1)) +
                      sizeof(uint64_t) * kTileTokens + sizeof(uint16_t) * (static_cast<size_t>(kLayoutWaves) * E + 2);
   hipLaunchKernelGGL(ep_layout_fused_kernel, dim3(a.num_tiles), dim3(kLayoutThreads), lds, stream, a);
   return hipGetLastError();

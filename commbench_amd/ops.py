@@ -81,6 +81,7 @@ class DispatchHandle:
     psum_rank_rows: torch.Tensor           # int32[R], inclusive rows per partition
     channel_prefix_matrix: Optional[torch.Tensor]  # int32[R, C]
     slot_rel: torch.Tensor                 # int32[T, K]
+    rank_slot_idx: Optional[torch.Tensor] = None   # int32[T, K], the prologue's dst_buffer_slot_idx
     slot_map: Optional[torch.Tensor] = None        # int32[T, K]
     recv_src_map: Optional[torch.Tensor] = None    # int32[capacity]
     recv_topk_idx: Optional[torch.Tensor] = None   # int64[capacity]
@@ -123,8 +124,12 @@ class Buffer:
                        "mi_ep_workspace_status")
 
     def dispatch_layout(self, topk_idx: torch.Tensor, expert_alignment: int = 1,
-                        num_channels: int = 0) -> DispatchHandle:
-        """Fused single-pass layout: counts, flags, offsets, per-route segment positions."""
+                        num_channels: int = 0, rank_slot_base: Optional[int] = None) -> DispatchHandle:
+        """Fused single-pass layout: counts, flags, offsets, per-route segment positions.
+
+        With `rank_slot_base` (the reference's scaleup_rank_idx * num_max_tokens_per_rank) the
+        handle also carries `rank_slot_idx`, the deterministic prologue's per-rank slot table
+        (example078 .cu:36-40)."""
         T, K = _check_routing(topk_idx, self.num_experts, self.num_ranks)
         _require(K == self.num_topk, "num_topk differs from the buffer's")
         _require(T <= self.num_max_tokens, "more tokens than the buffer was sized for")
@@ -140,14 +145,16 @@ class Buffer:
             channel_prefix_matrix=(torch.empty((R, num_channels), dtype=torch.int32, device=dev)
                                    if num_channels > 0 else None),
             slot_rel=torch.empty((T, K), dtype=torch.int32, device=dev),
+            rank_slot_idx=(torch.empty((T, K), dtype=torch.int32, device=dev)
+                           if rank_slot_base is not None else None),
         )
         lib = _lib.load()
         _lib.check(lib.mi_ep_dispatch_layout(
             _ptr(topk_idx), T, K, R, E, expert_alignment, num_channels,
             _ptr(h.num_tokens_per_rank), _ptr(h.num_tokens_per_expert), _ptr(h.is_token_in_rank),
             _ptr(h.expert_offsets), _ptr(h.psum_rank_rows), _ptr(h.channel_prefix_matrix),
-            _ptr(h.slot_rel), _ptr(self.workspace), self.workspace.numel(), _stream()),
-            "mi_ep_dispatch_layout")
+            _ptr(h.slot_rel), _ptr(h.rank_slot_idx), rank_slot_base or 0, _ptr(self.workspace),
+            self.workspace.numel(), _stream()), "mi_ep_dispatch_layout")
         return h
 
     def dispatch(self, x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Tensor,

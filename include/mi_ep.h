@@ -82,7 +82,7 @@ int mi_ep_set_wait_limit(unsigned int max_polls);
  *   example078 (deterministic slots, empty_deepep_jit_dispatch_deterministic_prologue.cu:27-43),
  *   example080 notify role (histogram, aligned exclusive expert psum, inclusive rank
  *   psum, empty_deepep_jit_dispatch_payload.cu:78-107,197-239).
- * Outputs (any of the last four may be NULL):
+ * Outputs (any of the last five may be NULL):
  *   num_tokens_per_rank / num_tokens_per_expert / is_token_in_rank   as above
  *   expert_offsets      int32[num_experts + 1]; off[0] = 0,
  *                       off[e+1] = off[e] + round_up(count[e], expert_alignment)
@@ -91,13 +91,19 @@ int mi_ep_set_wait_limit(unsigned int max_polls);
  *                       token tiles 0..c (tile bounds as get_channel_task_range, :73-79)
  *   slot_rel            int32[num_tokens, num_topk]; position of route (t,k) inside its
  *                       expert segment in (token, slot) order, -1 for non-routes
+ *   rank_slot_idx       int32[num_tokens, num_topk]; the prologue's own output format
+ *                       (dst_buffer_slot_idx, example078 .cu:36-40): for the first slot of every
+ *                       distinct destination rank of a token, rank_slot_base + the number of
+ *                       earlier tokens sent to that rank; -1 for masked slots and for further
+ *                       slots on a rank the token already reaches.  rank_slot_base stands for
+ *                       scaleup_rank_idx * kNumMaxTokensPerRank.
  */
 int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
                           int num_experts, int expert_alignment, int num_channels,
                           int* num_tokens_per_rank, int* num_tokens_per_expert,
                           bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
-                          int* channel_prefix_matrix, int* slot_rel, void* workspace,
-                          size_t workspace_bytes, void* stream);
+                          int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
+                          int rank_slot_base, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Dispatch (permute): the payload role of dispatch_impl

@@ -154,7 +154,8 @@ class ExpertParallelBuffer {
     MI_EP_CHECK(mi_ep_dispatch_layout(d_topk_idx, num_tokens, num_topk_, num_ranks_, num_experts_,
                                       h_.expert_alignment, num_channels_, h_.num_tokens_per_rank,
                                       h_.num_tokens_per_expert, h_.is_token_in_rank, h_.expert_offsets,
-                                      h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel, workspace_,
+                                      h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel,
+                                      /*rank_slot_idx=*/nullptr, /*rank_slot_base=*/0, workspace_,
                                       workspace_bytes_, stream));
     return h_;
   }

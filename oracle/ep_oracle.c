@@ -17,6 +17,7 @@
  *                               empty_deepep_jit_dispatch_deterministic_prologue.cu:27-43
  *                               (deterministic slots: earlier work is the prefix),
  *                               generalised from destination ranks to expert segments
+ *   ep_oracle_rank_slots        example078 ... deterministic_prologue.cu:27-43, in its own output format
  *   ep_oracle_channel_prefix    example047_deepep_intranode_notify_dispatch/nv/
  *                               empty_deepep_intranode_notify_dispatch.cu:73-79,386-406
  *   ep_oracle_rank_prefix       same file :352-360
@@ -37,6 +38,7 @@
  *                    brute force (tests/test_oracle_layout.py)
  *   expert offsets   numpy cumsum; off[E] == N; partition sums
  *   slot maps        numpy stable argsort by expert id (the map IS a stable sort)
+ *   rank slots       numpy: exclusive cumsum of the rank flags + first-occurrence mask
  *   channel prefix   closed form for the reference's routeDst pattern
  *   rank prefix      numpy cumsum over axis 0
  *   permute          numpy fancy-index gather
@@ -172,6 +174,32 @@ int ep_oracle_slot_maps(const int64_t* topk_idx, int num_tokens, int num_topk, i
       if (slot_map) slot_map[i] = row;
       if (src_map) src_map[row] = t;
       if (src_k) src_k[row] = k;
+    }
+  }
+  return 0;
+}
+
+/*
+ * The deterministic prologue's own table (example078 .cu:36-40): per destination rank, tokens
+ * take slots in token order; out[t,k] = base + slot for the first slot k of token t that
+ * reaches the rank, -1 for non-routes and for further slots on the same rank.
+ */
+int ep_oracle_rank_slots(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
+                         int num_experts, int base, int* out) {
+  if (num_ranks <= 0 || num_ranks > EP_MAX_RANKS || num_experts % num_ranks != 0) return -22;
+  const int per_rank = num_experts / num_ranks;
+  int next_slot[EP_MAX_RANKS] = {0};
+  for (int t = 0; t < num_tokens; ++t) {
+    int taken[EP_MAX_RANKS] = {0};
+    for (int k = 0; k < num_topk; ++k) {
+      size_t i = (size_t)t * num_topk + k;
+      int64_t e = topk_idx[i];
+      out[i] = -1;
+      if (!route_valid(e, num_experts)) continue;
+      int r = (int)(e / per_rank);
+      if (taken[r]) continue;
+      taken[r] = 1;
+      out[i] = base + next_slot[r]++;
     }
   }
   return 0;

@@ -98,6 +98,16 @@ def slot_maps(topk_idx: np.ndarray, num_experts: int, off: np.ndarray):
     return slot_rel, slot_map, src_map, src_k
 
 
+def rank_slots(topk_idx: np.ndarray, num_ranks: int, num_experts: int, base: int = 0) -> np.ndarray:
+    topk_idx = _c(topk_idx, np.int64)
+    T, K = topk_idx.shape
+    out = np.empty((T, K), dtype=np.int32)
+    rc = _load().ep_oracle_rank_slots(_p(topk_idx), T, K, num_ranks, num_experts, base, _p(out))
+    if rc != 0:
+        raise ValueError(f"ep_oracle_rank_slots: {rc}")
+    return out
+
+
 def channel_prefix(flags: np.ndarray, num_channels: int) -> np.ndarray:
     flags = _c(flags, np.uint8)
     T, R = flags.shape

@@ -33,9 +33,12 @@ def garbage_like(t: torch.Tensor) -> torch.Tensor:
     return t.view(torch.uint8).fill_(0xA5)
 
 
+RANK_SLOT_BASE = 5 * 65536
+
+
 def run_fused_layout(buf: ops.Buffer, topk_idx_np, expert_alignment=1, num_channels=0):
     topk = torch.from_numpy(topk_idx_np).to(DEV)
-    h = buf.dispatch_layout(topk, expert_alignment, num_channels)
+    h = buf.dispatch_layout(topk, expert_alignment, num_channels, rank_slot_base=RANK_SLOT_BASE)
     torch.cuda.synchronize()
     buf.status()
     return topk, h
@@ -51,6 +54,9 @@ def check_layout_against_oracle(oracle, h, topk_np, R, E, align=1, channels=0):
     np.testing.assert_array_equal(h.expert_offsets.cpu().numpy(), off)
     np.testing.assert_array_equal(h.psum_rank_rows.cpu().numpy(), psum)
     np.testing.assert_array_equal(h.slot_rel.cpu().numpy(), slot_rel)
+    if h.rank_slot_idx is not None and topk_np.shape[0] > 0:
+        np.testing.assert_array_equal(h.rank_slot_idx.cpu().numpy(),
+                                      oracle.rank_slots(topk_np, R, E, RANK_SLOT_BASE))
     if channels:
         np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy(),
                                       oracle.channel_prefix(flags, channels))

@@ -50,7 +50,7 @@ def test_host_only_entry_points():
     assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 9, 2, 8, None) == -22
     assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 2, 3, 8, None) == -22
     assert lib.mi_ep_dispatch_layout(None, 4, 2, 2, 8, 0, 0, None, None, None, None, None, None,
-                                     None, None, 0, None) == -22     # alignment 0
+                                     None, None, 0, None, 0, None) == -22     # alignment 0
     assert lib.mi_ep_combine(None, 0, None, None, None, None, None, 4, 2, 12, None, None, None) == -22
     assert lib.mi_ep_dispatch(None, None, None, None, None, None, None, 4, 2, 8, 1, 24, 0,
                               None, None, None, None, None, None, 0, None) == -22   # 24 % 16 != 0

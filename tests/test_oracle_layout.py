@@ -253,3 +253,56 @@ def test_rank_prefix_vs_cumsum(oracle):
     for R in (1, 2, 4, 8):
         counts = rng.integers(0, 5000, size=(R, R)).astype(np.int32)
         np.testing.assert_array_equal(oracle.rank_prefix(counts), np.cumsum(counts, axis=0))
+
+
+# ---- the deterministic prologue's own table (example078 .cu:36-40) ---------------------------
+
+def np_rank_slots(topk, R, E, base):
+    """Library restatement: exclusive cumsum of the rank flags gives each token's slot per rank;
+    the first slot of the token on that rank carries it."""
+    T, K = topk.shape
+    P = E // R
+    valid = (topk >= 0) & (topk < E)
+    rank = np.where(valid, topk // P, -1)
+    flags = np.zeros((T, R), dtype=np.int64)
+    for r in range(R):
+        flags[:, r] = (rank == r).any(axis=1)
+    slot_of_token = np.cumsum(flags, axis=0) - flags                   # exclusive, per rank
+    out = np.full((T, K), -1, dtype=np.int32)
+    for k in range(K):
+        first = valid[:, k] & ~(rank[:, :k] == rank[:, k:k + 1]).any(axis=1)
+        rows = np.nonzero(first)[0]
+        out[rows, k] = base + slot_of_token[rows, rank[rows, k]]
+    return out
+
+
+@pytest.mark.parametrize("case", wl.REFERENCE_LAYOUT_CASES[::2] + [(300, 8, 8, 64, "masked")],
+                         ids=lambda c: "-".join(map(str, c)))
+def test_rank_slots(oracle, case):
+    T, K, R, E, pattern = case
+    if pattern == "masked":
+        rng = np.random.default_rng(4)
+        topk = rng.integers(-2, E + 1, size=(T, K)).astype(np.int64)
+    else:
+        topk = wl.reference_pattern_topk(T, K, R, E, pattern)
+    base = 7 * 4096
+    got = oracle.rank_slots(topk, R, E, base)
+    np.testing.assert_array_equal(got, np_rank_slots(topk, R, E, base))
+    per_rank, _, flags = oracle.layout(topk, R, E)
+    P = E // R
+    for r in range(R):
+        on_r = (got >= 0) & (np.where((topk >= 0) & (topk < E), topk // P, -1) == r)
+        vals = got[on_r] - base
+        assert np.array_equal(vals, np.arange(per_rank[r]))             # token order, no gaps
+        assert np.array_equal(on_r.any(axis=1), flags[:, r].astype(bool))
+        assert on_r.sum(axis=1).max(initial=0) <= 1                      # one slot per (token, rank)
+
+
+def test_rank_slots_same_rank_case_by_hand(oracle):
+    # same_rank, K = 8: all eight slots of token t go to rank (3t + 8) mod R; only slot 0 carries it.
+    topk = wl.reference_pattern_topk(64, 8, 4, 16, "same_rank")
+    got = oracle.rank_slots(topk, 4, 16, 0)
+    assert (got[:, 1:] == -1).all()
+    # rank of token t is 3t mod 4: tokens 0, 4, 8, ... share rank 0 and take slots 0, 1, 2, ...
+    assert got[0, 0] == 0 and got[4, 0] == 1 and got[8, 0] == 2
+    assert got[1, 0] == 0 and got[5, 0] == 1                              # rank 3
