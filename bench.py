@@ -84,6 +84,7 @@ class Workload:
         self.psum = torch.empty(R, **i32)
         self.slot_rel = torch.empty((T, K), **i32)
         self.slot_map = torch.empty((T, K), **i32)
+        self.route_order = torch.empty((self.lib.mi_ep_route_order_bytes(T, K) // 16, 4), **i32)
         self.src_map = torch.empty(cap, **i32)
         self.recv_idx = torch.empty(cap, dtype=torch.int64, device=dev)
         self.recv_w = torch.empty(cap, dtype=torch.float32, device=dev)
@@ -101,7 +102,7 @@ class Workload:
             self.topk.data_ptr(), c.num_tokens, c.num_topk, c.num_ranks, c.num_experts, 1, 0,
             self.per_rank.data_ptr(), self.per_expert.data_ptr(), self.in_rank.data_ptr(),
             self.off.data_ptr(), self.psum.data_ptr(), None, self.slot_rel.data_ptr(), None, 0,
-            self.ws.data_ptr(), self.ws.numel(), self.stream), "layout")
+            self.route_order.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream), "layout")
 
     def dispatch(self):
         c = self.cfg
@@ -110,7 +111,7 @@ class Workload:
         self._lib.check(self.lib.mi_ep_dispatch(
             x.data_ptr(), None if self.scales is None else self.scales.data_ptr(),
             self.topk.data_ptr(), self.w.data_ptr(), self.off.data_ptr(), self.slot_rel.data_ptr(),
-            self.per_expert.data_ptr(), c.num_tokens, c.num_topk, c.num_experts, 1, c.row_bytes,
+            self.route_order.data_ptr(), self.per_expert.data_ptr(), c.num_tokens, c.num_topk, c.num_experts, 1, c.row_bytes,
             c.num_scales, self.recv_x.data_ptr(),
             None if self.recv_scales is None else self.recv_scales.data_ptr(),
             self.src_map.data_ptr(), self.recv_idx.data_ptr(), self.recv_w.data_ptr(),

@@ -36,6 +36,7 @@ inline int status_of(hipError_t e) { return e == hipSuccess ? MI_EP_OK : static_
 // so a few seconds before a launch gives up and flags the workspace.
 constexpr uint32_t kSpinLimit = 1u << 22;
 std::atomic<uint32_t> g_spin_limit{kSpinLimit};  // only ever changed by the test hook
+std::atomic<int> g_permute_schedule{kPermuteAuto};
 
 }  // namespace
 
@@ -92,6 +93,18 @@ int mi_ep_workspace_status(const void* workspace, void* stream) {
   return header.timed_out != 0 ? MI_EP_ETIMEDOUT : MI_EP_OK;
 }
 
+int mi_ep_set_dispatch_schedule(int schedule) {
+  if (schedule != kPermuteAuto && schedule != kPermuteByToken && schedule != kPermuteByDestination)
+    return MI_EP_EINVAL;
+  g_permute_schedule.store(schedule, std::memory_order_relaxed);
+  return MI_EP_OK;
+}
+
+size_t mi_ep_route_order_bytes(int num_tokens, int num_topk) {
+  if (num_tokens <= 0 || num_topk <= 0) return 0;
+  return static_cast<size_t>(num_tiles_for(num_tokens)) * kTileTokens * num_topk * 4 * sizeof(int);
+}
+
 int mi_ep_set_wait_limit(unsigned int max_polls) {
   g_spin_limit.store(max_polls == 0 ? kSpinLimit : max_polls, std::memory_order_relaxed);
   return MI_EP_OK;
@@ -102,7 +115,8 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
                           int* num_tokens_per_rank, int* num_tokens_per_expert,
                           bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
                           int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
-                          int rank_slot_base, void* workspace, size_t workspace_bytes, void* stream) {
+                          int rank_slot_base, int* route_order, void* workspace,
+                          size_t workspace_bytes, void* stream) {
   if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
   if (expert_alignment < 1) return MI_EP_EINVAL;
   if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
@@ -131,6 +145,7 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
 
   if (topk_idx == nullptr || is_token_in_rank == nullptr || workspace == nullptr) return MI_EP_EINVAL;
   if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
+  if (!aligned16(route_order)) return MI_EP_EINVAL;
   if (workspace_bytes < mi_ep_workspace_bytes(num_tokens, num_topk, num_experts, num_ranks))
     return MI_EP_ENOSPC;
 
@@ -145,6 +160,7 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
   a.slot_rel = slot_rel;
   a.rank_slot_idx = rank_slot_idx;
   a.rank_slot_base = rank_slot_base;
+  a.route_order = route_order;
   a.ws = static_cast<LayoutWorkspace*>(workspace);
   a.num_tokens = num_tokens;
   a.num_topk = num_topk;
@@ -164,7 +180,7 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
 
 int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
                    const float* topk_weights, const int* expert_offsets, const int* slot_rel,
-                   const int* num_tokens_per_expert, int num_tokens, int num_topk,
+                   const int* route_order, const int* num_tokens_per_expert, int num_tokens, int num_topk,
                    int num_experts, int expert_alignment, int row_bytes, int num_scales,
                    void* recv_x, float* recv_scales, int* recv_src_map, int64_t* recv_topk_idx,
                    float* recv_topk_weights, int* slot_map, int capacity_rows, void* stream) {
@@ -173,7 +189,7 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
   if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
   if (expert_offsets == nullptr || recv_src_map == nullptr) return MI_EP_EINVAL;
   if (capacity_rows > 0 && recv_x == nullptr) return MI_EP_EINVAL;
-  if (!aligned16(x) || !aligned16(recv_x)) return MI_EP_EINVAL;
+  if (!aligned16(x) || !aligned16(recv_x) || !aligned16(route_order)) return MI_EP_EINVAL;
   if (num_tokens > 0 &&
       (x == nullptr || topk_idx == nullptr || slot_rel == nullptr || slot_map == nullptr))
     return MI_EP_EINVAL;
@@ -188,6 +204,7 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
   a.topk_weights = topk_weights;
   a.expert_offsets = expert_offsets;
   a.slot_rel = slot_rel;
+  a.route_order = route_order;
   a.num_tokens_per_expert = num_tokens_per_expert;
   a.recv_x = static_cast<vec16*>(recv_x);
   a.recv_scales = recv_scales;
@@ -202,7 +219,7 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
   a.num_scales = num_scales;
   a.capacity_rows = capacity_rows;
   hipStream_t s = as_stream(stream);
-  hipError_t e = launch_permute(a, s);
+  hipError_t e = launch_permute(a, g_permute_schedule.load(std::memory_order_relaxed), s);
   if (e == hipSuccess && expert_alignment > 1) e = launch_pad_rows(a, s);
   return status_of(e);
 }

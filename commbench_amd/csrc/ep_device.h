@@ -41,6 +41,7 @@ struct LayoutArgs {
   int* channel_prefix_matrix;
   int* slot_rel;
   int* rank_slot_idx;
+  int* route_order;  // [num_tiles * kTileTokens * K][4] or null
   LayoutWorkspace* ws;
   int num_tokens;
   int num_topk;
@@ -72,6 +73,7 @@ struct PermuteArgs {
   const float* topk_weights;
   const int* expert_offsets;
   const int* slot_rel;
+  const int* route_order;  // the layout kernel's per-tile destination order, or null
   const int* num_tokens_per_expert;
   vec16* recv_x;
   float* recv_scales;
@@ -87,7 +89,11 @@ struct PermuteArgs {
   int capacity_rows;
 };
 
-hipError_t launch_permute(const PermuteArgs& a, hipStream_t stream);
+// Which copy kernel serves mi_ep_dispatch: chosen by shape, or forced (tests, measurements).
+constexpr int kPermuteAuto = 0;
+constexpr int kPermuteByToken = 1;        // wave per (token, 1 KiB): source read once, rows scattered
+constexpr int kPermuteByDestination = 2;  // needs route_order: rows written in destination order
+hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream);
 hipError_t launch_gather_rows(const vec16* x, const float* x_scales, const int* recv_src_map, int num_rows,
                               int num_tokens, int row_vecs, int num_scales, vec16* recv_x,
                               float* recv_scales, hipStream_t stream);

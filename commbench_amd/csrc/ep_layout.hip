@@ -86,7 +86,9 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   int* wave_sums = rank_cnt + kMaxRanks;    // [kLayoutWaves]
   int* misc = wave_sums + kLayoutWaves;     // [4] tile, generation
   int* rank_wave = misc + 4;                // [kTileTokens / kWave][kMaxRanks] flagged tokens per wave
-  int* offs = rank_wave + (kTileTokens / kWave) * kMaxRanks;  // [E + 2] offsets staged by the last tile
+  int* order_sums = rank_wave + (kTileTokens / kWave) * kMaxRanks;  // [kLayoutWaves] scan of the tile's counts
+  int* masked_wave = order_sums + kLayoutWaves;                      // [kLayoutWaves] non-routes per wave
+  int* offs = masked_wave + kLayoutWaves;   // [E + 2] per-expert bases: of the tile's route order, then of the segments
   uint64_t* tok_flags = reinterpret_cast<uint64_t*>(offs + E + 2 + (E & 1));  // [kTileTokens], byte r = rank r
   uint16_t* hist = reinterpret_cast<uint16_t*>(tok_flags + kTileTokens);  // [kLayoutWaves][E] wave-private
 
@@ -138,7 +140,8 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     }
   }
   int my_e[kChunksPerWave];
-  int my_pos[kChunksPerWave];
+  int my_pos[kChunksPerWave];  // rank among the wave's earlier routes to the same expert (among its non-routes if masked)
+  int masked_seen = 0;
 #pragma unroll
   for (int c = 0; c < kChunksPerWave; ++c) {
     my_e[c] = -1;
@@ -150,6 +153,10 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
       const bool valid = e64 >= 0 && e64 < static_cast<int64_t>(E);
       const int e = valid ? static_cast<int>(e64) : 0;
       const uint64_t same = match_expert(valid, e, a.expert_bits);
+      const bool masked = !valid && flat0 + local < flat_end;
+      const uint64_t masked_lanes = __ballot(masked);
+      if (masked) my_pos[c] = masked_seen + __popcll(masked_lanes & lanes_below(lane));
+      masked_seen += __popcll(masked_lanes);
       int old = 0, below = 0;
       if (valid) {
         below = __popcll(same & lanes_below(lane));
@@ -166,6 +173,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
       __builtin_amdgcn_wave_barrier();
     }
   }
+  if (lane == 0) masked_wave[wave] = masked_seen;
   __syncthreads();
 
   // ---- expert columns: wave bases, tile total, aggregate published at once ------
@@ -265,6 +273,50 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
         }
       }
     }
+  }
+
+  // ---- the tile's routes in destination order: by (expert, position in segment), then the
+  // non-routes in (token, slot) order.  Entry = {flat route index, expert, position, token}.
+  if (a.route_order != nullptr) {
+    const int local = tid < E ? col_total[tid] : 0;
+    int incl = local;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int up = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl += up;
+    }
+    if (lane == kWave - 1) order_sums[wave] = incl;
+    __syncthreads();
+    int base = incl - local;
+    int masked_base = 0;
+#pragma unroll
+    for (int w = 0; w < kLayoutWaves; ++w) {
+      if (w < wave) base += order_sums[w];
+      masked_base += order_sums[w];              // every route of the tile comes first
+      if (w < wave) masked_base += masked_wave[w];
+    }
+    if (tid < E) offs[tid] = base;
+    __syncthreads();
+    int4* order = reinterpret_cast<int4*>(a.route_order) + static_cast<size_t>(tile) * (kTileTokens * K);
+#pragma unroll
+    for (int c = 0; c < kChunksPerWave; ++c) {
+      const int chunk = wave * per_wave + c;
+      if (c < per_wave && chunk < num_chunks) {
+        const int g = flat0 + chunk * kWave + lane;
+        if (g < flat_end) {
+          const int e = my_e[c];
+          const int local = chunk * kWave + lane;
+          const int token = t0 + static_cast<int>((static_cast<uint32_t>(local) * a.inv_topk) >> 19);
+          if (e >= 0) {
+            const int in_tile = my_hist[e] + my_pos[c];
+            order[offs[e] + in_tile] = make_int4(g, e, col_excl[e] + in_tile, token);
+          } else {
+            order[masked_base + my_pos[c]] = make_int4(g, -1, -1, token);
+          }
+        }
+      }
+    }
+    __syncthreads();  // offs is reused by the last tile below
   }
 
   // ---- the deterministic prologue's table: per destination rank, tokens take slots in
@@ -469,7 +521,7 @@ hipError_t launch_layout_fused(const LayoutArgs& a, hipStream_t stream) {
   const int E = a.num_experts;
   const int cols = E + a.num_ranks;
   const size_t lds = sizeof(int) * (2 * static_cast<size_t>(cols) + kMaxRanks + kLayoutWaves + 4 +
-                                    (kTileTokens / kWave) * kMaxRanks + E + 2 + (E & 1)) +
+                                    (kTileTokens / kWave) * kMaxRanks + 2 * kLayoutWaves + E + 2 + (E & 1)) +
                      sizeof(uint64_t) * kTileTokens + sizeof(uint16_t) * (static_cast<size_t>(kLayoutWaves) * E + 2);
   hipLaunchKernelGGL(ep_layout_fused_kernel, dim3(a.num_tiles), dim3(kLayoutThreads), lds, stream, a);
   return hipGetLastError();

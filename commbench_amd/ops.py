@@ -82,6 +82,7 @@ class DispatchHandle:
     channel_prefix_matrix: Optional[torch.Tensor]  # int32[R, C]
     slot_rel: torch.Tensor                 # int32[T, K]
     rank_slot_idx: Optional[torch.Tensor] = None   # int32[T, K], the prologue's dst_buffer_slot_idx
+    route_order: Optional[torch.Tensor] = None     # int32[tiles * 256 * K, 4], routes in destination order
     slot_map: Optional[torch.Tensor] = None        # int32[T, K]
     recv_src_map: Optional[torch.Tensor] = None    # int32[capacity]
     recv_topk_idx: Optional[torch.Tensor] = None   # int64[capacity]
@@ -124,8 +125,11 @@ class Buffer:
                        "mi_ep_workspace_status")
 
     def dispatch_layout(self, topk_idx: torch.Tensor, expert_alignment: int = 1,
-                        num_channels: int = 0, rank_slot_base: Optional[int] = None) -> DispatchHandle:
-        """Fused single-pass layout: counts, flags, offsets, per-route segment positions.
+                        num_channels: int = 0, rank_slot_base: Optional[int] = None,
+                        route_order: bool = True) -> DispatchHandle:
+        """Fused single-pass layout: counts, flags, offsets, per-route segment positions, and
+        (unless `route_order` is False) the per-tile destination order that lets dispatch write
+        adjacent rows together.
 
         With `rank_slot_base` (the reference's scaleup_rank_idx * num_max_tokens_per_rank) the
         handle also carries `rank_slot_idx`, the deterministic prologue's per-rank slot table
@@ -149,11 +153,15 @@ class Buffer:
                            if rank_slot_base is not None else None),
         )
         lib = _lib.load()
+        if route_order and T > 0:
+            h.route_order = torch.empty((lib.mi_ep_route_order_bytes(T, K) // 16, 4), dtype=torch.int32,
+                                        device=dev)
         _lib.check(lib.mi_ep_dispatch_layout(
             _ptr(topk_idx), T, K, R, E, expert_alignment, num_channels,
             _ptr(h.num_tokens_per_rank), _ptr(h.num_tokens_per_expert), _ptr(h.is_token_in_rank),
             _ptr(h.expert_offsets), _ptr(h.psum_rank_rows), _ptr(h.channel_prefix_matrix),
-            _ptr(h.slot_rel), _ptr(h.rank_slot_idx), rank_slot_base or 0, _ptr(self.workspace),
+            _ptr(h.slot_rel), _ptr(h.rank_slot_idx), rank_slot_base or 0, _ptr(h.route_order),
+            _ptr(self.workspace),
             self.workspace.numel(), _stream()), "mi_ep_dispatch_layout")
         return h
 
@@ -196,7 +204,7 @@ class Buffer:
         lib = _lib.load()
         _lib.check(lib.mi_ep_dispatch(
             _ptr(x), _ptr(scales), _ptr(topk_idx), _ptr(topk_weights), _ptr(handle.expert_offsets),
-            _ptr(handle.slot_rel), _ptr(handle.num_tokens_per_expert), T, K, E,
+            _ptr(handle.slot_rel), _ptr(handle.route_order), _ptr(handle.num_tokens_per_expert), T, K, E,
             handle.expert_alignment, row_bytes, num_scales, _ptr(recv_x), _ptr(recv_scales),
             _ptr(handle.recv_src_map), _ptr(handle.recv_topk_idx), _ptr(handle.recv_topk_weights),
             _ptr(handle.slot_map), capacity_rows, _stream()), "mi_ep_dispatch")

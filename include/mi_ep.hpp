@@ -93,6 +93,7 @@ struct DispatchHandle {
   int* psum_rank_rows = nullptr;         // [R]
   int* channel_prefix_matrix = nullptr;  // [R, C] (C = num_channels of the buffer, may be 0)
   int* slot_rel = nullptr;               // [T, K]
+  int* route_order = nullptr;            // [tiles * 256 * K, 4] routes in destination order
   int* slot_map = nullptr;               // [T, K]
   int* recv_src_map = nullptr;           // [capacity]
   int64_t* recv_topk_idx = nullptr;      // [capacity]
@@ -125,6 +126,7 @@ class ExpertParallelBuffer {
     if (num_channels > 0)
       MI_EP_HIP_CHECK(hipMalloc(&h_.channel_prefix_matrix, sizeof(int) * num_ranks * num_channels));
     MI_EP_HIP_CHECK(hipMalloc(&h_.slot_rel, sizeof(int) * (tk + 1)));
+    MI_EP_HIP_CHECK(hipMalloc(&h_.route_order, mi_ep_route_order_bytes(num_max_tokens, num_topk) + 16));
     MI_EP_HIP_CHECK(hipMalloc(&h_.slot_map, sizeof(int) * (tk + 1)));
     MI_EP_HIP_CHECK(hipMalloc(&h_.recv_src_map, sizeof(int) * (capacity_ + 1)));
     MI_EP_HIP_CHECK(hipMalloc(&h_.recv_topk_idx, sizeof(int64_t) * (capacity_ + 1)));
@@ -136,7 +138,7 @@ class ExpertParallelBuffer {
   ~ExpertParallelBuffer() {
     void* owned[] = {workspace_, h_.num_tokens_per_rank, h_.num_tokens_per_expert, h_.is_token_in_rank,
                      h_.expert_offsets, h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel,
-                     h_.slot_map, h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights};
+                     h_.route_order, h_.slot_map, h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights};
     for (void* p : owned)
       if (p != nullptr) (void)hipFree(p);
   }
@@ -155,8 +157,8 @@ class ExpertParallelBuffer {
                                       h_.expert_alignment, num_channels_, h_.num_tokens_per_rank,
                                       h_.num_tokens_per_expert, h_.is_token_in_rank, h_.expert_offsets,
                                       h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel,
-                                      /*rank_slot_idx=*/nullptr, /*rank_slot_base=*/0, workspace_,
-                                      workspace_bytes_, stream));
+                                      /*rank_slot_idx=*/nullptr, /*rank_slot_base=*/0, h_.route_order,
+                                      workspace_, workspace_bytes_, stream));
     return h_;
   }
 
@@ -166,7 +168,7 @@ class ExpertParallelBuffer {
                                  void* d_recv_x, float* d_recv_scales, hipStream_t stream = 0) {
     get_dispatch_layout(d_topk_idx, num_tokens, stream);
     MI_EP_CHECK(mi_ep_dispatch(d_x, d_scales, d_topk_idx, d_topk_weights, h_.expert_offsets, h_.slot_rel,
-                               h_.num_tokens_per_expert, num_tokens, num_topk_, num_experts_,
+                               h_.route_order, h_.num_tokens_per_expert, num_tokens, num_topk_, num_experts_,
                                h_.expert_alignment, row_bytes, num_scales, d_recv_x, d_recv_scales,
                                h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights, h_.slot_map,
                                capacity_, stream));

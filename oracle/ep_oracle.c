@@ -18,6 +18,8 @@
  *                               (deterministic slots: earlier work is the prefix),
  *                               generalised from destination ranks to expert segments
  *   ep_oracle_rank_slots        example078 ... deterministic_prologue.cu:27-43, in its own output format
+ *   ep_oracle_route_order       no reference kernel: the per-tile stable sort of routes by expert that
+ *                               the destination-order copy walks (nearest relative: example056 :521-564)
  *   ep_oracle_channel_prefix    example047_deepep_intranode_notify_dispatch/nv/
  *                               empty_deepep_intranode_notify_dispatch.cu:73-79,386-406
  *   ep_oracle_rank_prefix       same file :352-360
@@ -39,6 +41,7 @@
  *   expert offsets   numpy cumsum; off[E] == N; partition sums
  *   slot maps        numpy stable argsort by expert id (the map IS a stable sort)
  *   rank slots       numpy: exclusive cumsum of the rank flags + first-occurrence mask
+ *   route order      numpy lexsort per tile; positions agree with the slot maps
  *   channel prefix   closed form for the reference's routeDst pattern
  *   rank prefix      numpy cumsum over axis 0
  *   permute          numpy fancy-index gather
@@ -200,6 +203,54 @@ int ep_oracle_rank_slots(const int64_t* topk_idx, int num_tokens, int num_topk, 
       if (taken[r]) continue;
       taken[r] = 1;
       out[i] = base + next_slot[r]++;
+    }
+  }
+  return 0;
+}
+
+/*
+ * Routes of every tile of `tile_tokens` consecutive tokens in destination order: a stable
+ * counting sort of the tile's routes by expert (so by position in the expert's segment),
+ * non-routes after them in (token, slot) order.  Entry i of tile j sits at
+ * out[(j * tile_tokens * K + i) * 4 ..] = {t*K + k, expert, slot_rel, t}, with expert and
+ * slot_rel -1 for non-routes; entries past the last token's are left untouched.  This is the
+ * sender-side counterpart of the sorted pull list the ThunderKittens example builds
+ * (example056 compute_dispatch_indices, :521-564), restricted to one tile.
+ * `scratch` holds 2 * num_experts ints.
+ */
+int ep_oracle_route_order(const int64_t* topk_idx, int num_tokens, int num_topk, int num_experts,
+                          int tile_tokens, int* out, int* scratch) {
+  if (tile_tokens <= 0) return -22;
+  int* seen = scratch;                 /* routes of expert e in earlier tokens */
+  int* next = scratch + num_experts;   /* next position of expert e inside the tile's list */
+  memset(seen, 0, sizeof(int) * (size_t)num_experts);
+  for (int t0 = 0; t0 < num_tokens; t0 += tile_tokens) {
+    const int t1 = t0 + tile_tokens < num_tokens ? t0 + tile_tokens : num_tokens;
+    int* list = out + (size_t)(t0 / tile_tokens) * tile_tokens * num_topk * 4;
+    memset(next, 0, sizeof(int) * (size_t)num_experts);
+    for (size_t i = (size_t)t0 * num_topk; i < (size_t)t1 * num_topk; ++i)
+      if (route_valid(topk_idx[i], num_experts)) next[topk_idx[i]]++;
+    int total = 0;
+    for (int e = 0; e < num_experts; ++e) {
+      int c = next[e];
+      next[e] = total;
+      total += c;
+    }
+    int masked = total;
+    for (size_t i = (size_t)t0 * num_topk; i < (size_t)t1 * num_topk; ++i) {
+      int64_t e = topk_idx[i];
+      int* entry;
+      if (route_valid(e, num_experts)) {
+        entry = list + 4 * (size_t)next[e]++;
+        entry[1] = (int)e;
+        entry[2] = seen[e]++;
+      } else {
+        entry = list + 4 * (size_t)masked++;
+        entry[1] = -1;
+        entry[2] = -1;
+      }
+      entry[0] = (int)i;
+      entry[3] = (int)(i / (size_t)num_topk);
     }
   }
   return 0;

@@ -108,6 +108,19 @@ def rank_slots(topk_idx: np.ndarray, num_ranks: int, num_experts: int, base: int
     return out
 
 
+def route_order(topk_idx: np.ndarray, num_experts: int, tile_tokens: int = 256, fill: int = -7) -> np.ndarray:
+    """int32[tiles * tile_tokens * K, 4]; entries past the last token's keep `fill`."""
+    topk_idx = _c(topk_idx, np.int64)
+    T, K = topk_idx.shape
+    tiles = (T + tile_tokens - 1) // tile_tokens
+    out = np.full((tiles * tile_tokens * K, 4), fill, dtype=np.int32)
+    scratch = np.empty(2 * num_experts, dtype=np.int32)
+    rc = _load().ep_oracle_route_order(_p(topk_idx), T, K, num_experts, tile_tokens, _p(out), _p(scratch))
+    if rc != 0:
+        raise ValueError(f"ep_oracle_route_order: {rc}")
+    return out
+
+
 def channel_prefix(flags: np.ndarray, num_channels: int) -> np.ndarray:
     flags = _c(flags, np.uint8)
     T, R = flags.shape

@@ -34,6 +34,8 @@ def garbage_like(t: torch.Tensor) -> torch.Tensor:
 
 
 RANK_SLOT_BASE = 5 * 65536
+SCHEDULE_AUTO, SCHEDULE_BY_TOKEN, SCHEDULE_BY_DESTINATION = 0, 1, 2   # mi_ep_set_dispatch_schedule
+TILE_TOKENS = 256                                                     # tokens per route_order tile
 
 
 def run_fused_layout(buf: ops.Buffer, topk_idx_np, expert_alignment=1, num_channels=0):
@@ -57,6 +59,12 @@ def check_layout_against_oracle(oracle, h, topk_np, R, E, align=1, channels=0):
     if h.rank_slot_idx is not None and topk_np.shape[0] > 0:
         np.testing.assert_array_equal(h.rank_slot_idx.cpu().numpy(),
                                       oracle.rank_slots(topk_np, R, E, RANK_SLOT_BASE))
+    if h.route_order is not None and topk_np.shape[0] > 0:
+        want = oracle.route_order(topk_np, E, TILE_TOKENS)
+        got = h.route_order.cpu().numpy()
+        assert got.shape == want.shape
+        written = want[:, 0] != -7                       # entries past the last token are unspecified
+        np.testing.assert_array_equal(got[written], want[written])
     if channels:
         np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy(),
                                       oracle.channel_prefix(flags, channels))

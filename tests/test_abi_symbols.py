@@ -42,6 +42,11 @@ def test_host_only_entry_points():
     # 256-byte header + ceil(T/256) tiles x (E + R) 8-byte status words
     assert lib.mi_ep_workspace_bytes(8192, 8, 256, 8) == 256 + 32 * 264 * 8
     assert lib.mi_ep_workspace_bytes(1, 1, 1, 1) == 256 + 1 * 2 * 8
+    # one 16-byte entry per route slot of every 256-token tile
+    assert lib.mi_ep_route_order_bytes(8192, 8) == 32 * 256 * 8 * 16
+    assert lib.mi_ep_route_order_bytes(257, 3) == 2 * 256 * 3 * 16
+    assert lib.mi_ep_route_order_bytes(0, 8) == 0
+    assert lib.mi_ep_set_dispatch_schedule(7) == -22 and lib.mi_ep_set_dispatch_schedule(0) == 0
     assert lib.mi_ep_workspace_bytes(8192, 8, 256, 9) == 0       # more than 8 ranks
     assert lib.mi_ep_workspace_bytes(8192, 9, 256, 8) == 0       # more than 8 slots
     assert lib.mi_ep_workspace_bytes(8192, 8, 250, 8) == 0       # experts not divisible by ranks
@@ -50,9 +55,9 @@ def test_host_only_entry_points():
     assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 9, 2, 8, None) == -22
     assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 2, 3, 8, None) == -22
     assert lib.mi_ep_dispatch_layout(None, 4, 2, 2, 8, 0, 0, None, None, None, None, None, None,
-                                     None, None, 0, None, 0, None) == -22     # alignment 0
+                                     None, None, 0, None, None, 0, None) == -22     # alignment 0
     assert lib.mi_ep_combine(None, 0, None, None, None, None, None, 4, 2, 12, None, None, None) == -22
-    assert lib.mi_ep_dispatch(None, None, None, None, None, None, None, 4, 2, 8, 1, 24, 0,
+    assert lib.mi_ep_dispatch(None, None, None, None, None, None, None, None, 4, 2, 8, 1, 24, 0,
                               None, None, None, None, None, None, 0, None) == -22   # 24 % 16 != 0
 
 

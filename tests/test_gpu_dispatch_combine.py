@@ -19,7 +19,9 @@ COMBINE_ULP_TOLERANCE = 2
 
 
 def dispatch_and_check(oracle, cfg_or_shape, topk_np, w_np, x_cpu, scales_cpu, align=1):
-    """Runs layout + permute on the GPU, compares everything with the checker, returns both."""
+    """Runs layout + permute on the GPU under both copy schedules (by token, by destination),
+    compares everything with the checker each time, returns the last run and the checker's."""
+    from commbench_amd import _lib
     T, K = topk_np.shape
     E, R = cfg_or_shape
     buf = ops.Buffer(T, K, E, R, device=gu.DEV)
@@ -27,23 +29,30 @@ def dispatch_and_check(oracle, cfg_or_shape, topk_np, w_np, x_cpu, scales_cpu, a
     w = torch.from_numpy(w_np).to(gu.DEV) if w_np is not None else None
     x = x_cpu.to(gu.DEV)
     scales = scales_cpu.to(gu.DEV) if scales_cpu is not None else None
-    recv_x, recv_scales, recv_src_map, h = buf.dispatch(x, scales, topk, w, expert_alignment=align)
-    torch.cuda.synchronize()
-    buf.status()
     ref = oracle.full_path(topk_np, w_np, gu.as_bytes(x_cpu),
                            None if scales_cpu is None else scales_cpu.numpy(), E, R, align)
     rows = int(ref["expert_offsets"][-1])
-    assert h.num_recv_rows() == rows
-    np.testing.assert_array_equal(h.slot_map.cpu().numpy(), ref["slot_map"])
-    np.testing.assert_array_equal(recv_src_map.cpu().numpy()[:rows], ref["recv_src_map"])
-    np.testing.assert_array_equal(h.recv_topk_idx.cpu().numpy()[:rows], ref["recv_topk_idx"])
-    np.testing.assert_array_equal(gu.as_bytes(recv_x)[:rows], ref["recv_x"])
-    if scales_cpu is not None:
-        np.testing.assert_array_equal(recv_scales.cpu().numpy()[:rows].view(np.uint32),
-                                      ref["recv_scales"].view(np.uint32))
-    if w_np is not None:
-        np.testing.assert_array_equal(h.recv_topk_weights.cpu().numpy()[:rows].view(np.uint32),
-                                      ref["recv_topk_weights"].view(np.uint32))
+    lib = _lib.load()
+    for schedule in (gu.SCHEDULE_BY_TOKEN, gu.SCHEDULE_BY_DESTINATION):
+        print(f"schedule {schedule}", flush=True)
+        assert lib.mi_ep_set_dispatch_schedule(schedule) == 0
+        try:
+            recv_x, recv_scales, recv_src_map, h = buf.dispatch(x, scales, topk, w, expert_alignment=align)
+            torch.cuda.synchronize()
+        finally:
+            assert lib.mi_ep_set_dispatch_schedule(gu.SCHEDULE_AUTO) == 0
+        buf.status()
+        assert h.num_recv_rows() == rows
+        np.testing.assert_array_equal(h.slot_map.cpu().numpy(), ref["slot_map"])
+        np.testing.assert_array_equal(recv_src_map.cpu().numpy()[:rows], ref["recv_src_map"])
+        np.testing.assert_array_equal(h.recv_topk_idx.cpu().numpy()[:rows], ref["recv_topk_idx"])
+        np.testing.assert_array_equal(gu.as_bytes(recv_x)[:rows], ref["recv_x"])
+        if scales_cpu is not None:
+            np.testing.assert_array_equal(recv_scales.cpu().numpy()[:rows].view(np.uint32),
+                                          ref["recv_scales"].view(np.uint32))
+        if w_np is not None:
+            np.testing.assert_array_equal(h.recv_topk_weights.cpu().numpy()[:rows].view(np.uint32),
+                                          ref["recv_topk_weights"].view(np.uint32))
     return recv_x, h, ref
 
 

@@ -27,6 +27,7 @@ def test_graph_replays_match_eager(oracle):
     in_rank = torch.empty((T, R), dtype=torch.bool, device=dev)
     off, psum = torch.empty(E + 1, **i32), torch.empty(R, **i32)
     slot_rel, slot_map = torch.empty((T, K), **i32), torch.empty((T, K), **i32)
+    route_order = torch.empty((lib.mi_ep_route_order_bytes(T, K) // 16, 4), **i32)
     src_map = torch.empty(cap, **i32)
     recv_idx = torch.empty(cap, dtype=torch.int64, device=dev)
     recv_w = torch.empty(cap, dtype=torch.float32, device=dev)
@@ -40,10 +41,10 @@ def test_graph_replays_match_eager(oracle):
         _lib.check(lib.mi_ep_dispatch_layout(
             topk.data_ptr(), T, K, R, E, 1, 0, per_rank.data_ptr(), per_expert.data_ptr(),
             in_rank.data_ptr(), off.data_ptr(), psum.data_ptr(), None, slot_rel.data_ptr(), None, 0,
-            ws.data_ptr(), ws_bytes, stream), "layout")
+            route_order.data_ptr(), ws.data_ptr(), ws_bytes, stream), "layout")
         _lib.check(lib.mi_ep_dispatch(
             x.data_ptr(), None, topk.data_ptr(), w.data_ptr(), off.data_ptr(), slot_rel.data_ptr(),
-            per_expert.data_ptr(), T, K, E, 1, H * 2, 0, recv_x.data_ptr(), None, src_map.data_ptr(),
+            route_order.data_ptr(), per_expert.data_ptr(), T, K, E, 1, H * 2, 0, recv_x.data_ptr(), None, src_map.data_ptr(),
             recv_idx.data_ptr(), recv_w.data_ptr(), slot_map.data_ptr(), cap, stream), "dispatch")
         _lib.check(lib.mi_ep_combine(
             recv_x.data_ptr(), cap, slot_map.data_ptr(), w.data_ptr(), None, None, None, T, K, H,

@@ -306,3 +306,71 @@ def test_rank_slots_same_rank_case_by_hand(oracle):
     # rank of token t is 3t mod 4: tokens 0, 4, 8, ... share rank 0 and take slots 0, 1, 2, ...
     assert got[0, 0] == 0 and got[4, 0] == 1 and got[8, 0] == 2
     assert got[1, 0] == 0 and got[5, 0] == 1                              # rank 3
+
+
+# ---- per-tile destination order of the routes -------------------------------------------------
+
+def np_route_order(topk, E, tile):
+    """Library restatement: inside a tile, routes by (expert, flat index) with numpy's lexsort,
+    then the non-routes by flat index; the position column comes from the slot maps."""
+    T, K = topk.shape
+    flat = topk.reshape(-1)
+    valid = (flat >= 0) & (flat < E)
+    counts = np.bincount(flat[valid], minlength=E)
+    off = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    tiles = (T + tile - 1) // tile
+    out = np.full((tiles * tile * K, 4), -7, dtype=np.int32)
+    # position inside the expert's segment = rank of the route among the expert's routes
+    order = np.argsort(np.where(valid, flat, E), kind="stable")
+    rel = np.full(T * K, -1, dtype=np.int64)
+    rel[order[:valid.sum()]] = np.arange(valid.sum()) - off[flat[order[:valid.sum()]]]
+    for j in range(tiles):
+        g = np.arange(j * tile * K, min((j + 1) * tile, T) * K)
+        v = valid[g]
+        routed = g[v][np.lexsort((g[v], flat[g[v]]))]
+        masked = g[~v]
+        base = j * tile * K
+        out[base:base + len(routed)] = np.stack(
+            [routed, flat[routed], rel[routed], routed // K], axis=1)
+        out[base + len(routed):base + len(g)] = np.stack(
+            [masked, -np.ones_like(masked), -np.ones_like(masked), masked // K], axis=1)
+    return out
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 4), (7, 2, 4, 4), (256, 8, 64, 256), (257, 3, 5, 256),
+                                   (1000, 8, 256, 256), (3000, 6, 1024, 256), (700, 4, 16, 64)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_route_order_vs_lexsort(oracle, shape):
+    T, K, E, tile = shape
+    rng = np.random.default_rng(T + K)
+    topk = rng.integers(-2, E + 2, size=(T, K)).astype(np.int64)       # masks, out of range, duplicates
+    got = oracle.route_order(topk, E, tile)
+    np.testing.assert_array_equal(got, np_route_order(topk, E, tile))
+    # every flat index exactly once; positions agree with the slot maps
+    written = got[got[:, 0] != -7]
+    assert np.array_equal(np.sort(written[:, 0]), np.arange(T * K))
+    _, per_expert, _ = oracle.layout(topk, 1, E)
+    off, _ = oracle.expert_offsets(per_expert, 1, 1)
+    slot_rel, _, _, _ = oracle.slot_maps(topk, E, off)
+    assert np.array_equal(written[:, 2], slot_rel.reshape(-1)[written[:, 0]])
+    # destination rows of a tile's routes ascend: that is what the copy kernel relies on
+    for j in range((T + tile - 1) // tile):
+        part = got[j * tile * K:(j + 1) * tile * K]
+        part = part[(part[:, 0] != -7) & (part[:, 1] >= 0)]
+        dst = off[part[:, 1]].astype(np.int64) + part[:, 2]
+        assert (np.diff(dst) > 0).all()
+
+
+def test_route_order_by_hand(oracle):
+    # 3 tokens x 2 slots, tile of 2 tokens, 3 experts.
+    topk = np.array([[2, 0], [-1, 2], [0, 0]], dtype=np.int64)
+    got = oracle.route_order(topk, 3, tile_tokens=2)
+    want = np.array([
+        [1, 0, 0, 0],      # tile 0: expert 0 <- route (0,1), first in its segment
+        [0, 2, 0, 0],      #         expert 2 <- route (0,0)
+        [3, 2, 1, 1],      #         expert 2 <- route (1,1), second in the segment
+        [2, -1, -1, 1],    #         the masked slot (1,0)
+        [4, 0, 1, 2],      # tile 1: expert 0 <- route (2,0), after tile 0's one
+        [5, 0, 2, 2],      #         expert 0 <- route (2,1)
+        [-7, -7, -7, -7], [-7, -7, -7, -7]], dtype=np.int32)
+    np.testing.assert_array_equal(got, want)
