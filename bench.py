@@ -365,14 +365,14 @@ def main():
                 continue
             ocfg = wl.CONFIGS[name]
             owk = Workload(ocfg, dev)
-            for _ in range(5):
+            for _ in range(10):
                 owk.step()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            for _ in range(20):
+            for _ in range(100):
                 owk.step()
             torch.cuda.synchronize()
-            us = (time.perf_counter() - t0) * 1e6 / 20
+            us = (time.perf_counter() - t0) * 1e6 / 100
             others[name] = {"us_per_step": us, "tokens_per_s": ocfg.num_tokens / (us * 1e-6),
                             "hbm_gbps_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9,
                             "hbm_frac_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS,
