@@ -178,7 +178,8 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
 
   // ---- expert columns: wave bases, tile total, aggregate published at once ------
   // (the status words need a few microseconds to reach the other tiles; the flag
-  // pass below runs in that shadow)
+  // pass and the scan for the tile's route order run in that shadow)
+  int my_col_total = 0;  // thread e < E: this tile's routes to expert e
   for (int col = tid; col < E; col += kLayoutThreads) {
     int total = 0;
 #pragma unroll
@@ -188,8 +189,20 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
       total += v;
     }
     col_total[col] = total;
+    my_col_total = total;
     publish(status + static_cast<size_t>(tile) * cols + col,
             pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
+  }
+  // Exclusive scan of the tile's per-expert counts (one expert per thread): where each expert's
+  // routes start in the tile's route order.  The cross-wave half follows the next barrier.
+  int order_incl = my_col_total;
+  if (a.route_order != nullptr) {
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int up = __shfl_up(order_incl, d, kWave);
+      if (lane >= d) order_incl += up;
+    }
+    if (lane == kWave - 1) order_sums[wave] = order_incl;
   }
 
   // ---- flags out, de-duplicated rank hits (one token per thread) ---------------
@@ -203,6 +216,18 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     }
   }
   __syncthreads();
+
+  int masked_base = 0;  // where this wave's non-routes start in the tile's route order
+  if (a.route_order != nullptr) {
+    int base = order_incl - my_col_total;
+#pragma unroll
+    for (int w = 0; w < kLayoutWaves; ++w) {
+      if (w < wave) base += order_sums[w];
+      masked_base += order_sums[w];  // every route of the tile comes first
+      if (w < wave) masked_base += masked_wave[w];
+    }
+    if (tid < E) offs[tid] = base;  // read after the barrier that ends the look-back
+  }
 
   // ---- rank columns published, then the decoupled look-back of every column ------
   for (int col = tid; col < cols; col += kLayoutThreads) {
@@ -260,63 +285,30 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   }
   __syncthreads();
 
-  // ---- position of every route inside its expert segment --------------------
-  if (a.slot_rel != nullptr) {
-#pragma unroll
-    for (int c = 0; c < kChunksPerWave; ++c) {
-      const int chunk = wave * per_wave + c;
-      if (c < per_wave && chunk < num_chunks) {
-        const int g = flat0 + chunk * kWave + lane;
-        if (g < flat_end) {
-          const int e = my_e[c];
-          a.slot_rel[g] = (e >= 0) ? col_excl[e] + my_hist[e] + my_pos[c] : -1;
-        }
-      }
-    }
-  }
-
-  // ---- the tile's routes in destination order: by (expert, position in segment), then the
-  // non-routes in (token, slot) order.  Entry = {flat route index, expert, position, token}.
-  if (a.route_order != nullptr) {
-    const int local = tid < E ? col_total[tid] : 0;
-    int incl = local;
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const int up = __shfl_up(incl, d, kWave);
-      if (lane >= d) incl += up;
-    }
-    if (lane == kWave - 1) order_sums[wave] = incl;
-    __syncthreads();
-    int base = incl - local;
-    int masked_base = 0;
-#pragma unroll
-    for (int w = 0; w < kLayoutWaves; ++w) {
-      if (w < wave) base += order_sums[w];
-      masked_base += order_sums[w];              // every route of the tile comes first
-      if (w < wave) masked_base += masked_wave[w];
-    }
-    if (tid < E) offs[tid] = base;
-    __syncthreads();
+  // ---- position of every route inside its expert segment, and the tile's routes in
+  // destination order: by (expert, position in segment), then the non-routes in (token, slot)
+  // order.  Entry = {flat route index, expert, position, token}.
+  if (a.slot_rel != nullptr || a.route_order != nullptr) {
     int4* order = reinterpret_cast<int4*>(a.route_order) + static_cast<size_t>(tile) * (kTileTokens * K);
 #pragma unroll
     for (int c = 0; c < kChunksPerWave; ++c) {
       const int chunk = wave * per_wave + c;
       if (c < per_wave && chunk < num_chunks) {
-        const int g = flat0 + chunk * kWave + lane;
+        const int local = chunk * kWave + lane;
+        const int g = flat0 + local;
         if (g < flat_end) {
           const int e = my_e[c];
-          const int local = chunk * kWave + lane;
-          const int token = t0 + static_cast<int>((static_cast<uint32_t>(local) * a.inv_topk) >> 19);
-          if (e >= 0) {
-            const int in_tile = my_hist[e] + my_pos[c];
-            order[offs[e] + in_tile] = make_int4(g, e, col_excl[e] + in_tile, token);
-          } else {
-            order[masked_base + my_pos[c]] = make_int4(g, -1, -1, token);
+          const int in_tile = (e >= 0) ? my_hist[e] + my_pos[c] : 0;
+          const int rel = (e >= 0) ? col_excl[e] + in_tile : -1;
+          if (a.slot_rel != nullptr) a.slot_rel[g] = rel;
+          if (a.route_order != nullptr) {
+            const int token = t0 + static_cast<int>((static_cast<uint32_t>(local) * a.inv_topk) >> 19);
+            const int pos = (e >= 0) ? offs[e] + in_tile : masked_base + my_pos[c];
+            order[pos] = make_int4(g, e, rel, token);
           }
         }
       }
     }
-    __syncthreads();  // offs is reused by the last tile below
   }
 
   // ---- the deterministic prologue's table: per destination rank, tokens take slots in
