@@ -271,7 +271,8 @@ def main():
     # (persistent LDS-staged kernel from 16 tokens per compute unit and 2 KiB rows upwards).
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     staged = T >= 16 * cus and 2048 <= cfg.hidden * 2 <= 160 * 1024
-    names = ["ep_layout_fused_kernel", "ep_permute_kernel",
+    by_destination = wk.lib.mi_ep_dispatch_schedule_for(T, cfg.num_topk, cfg.num_experts, cfg.row_bytes) == 2
+    names = ["ep_layout_fused_kernel", "ep_permute_tiles_kernel" if by_destination else "ep_permute_kernel",
              "ep_combine_staged_kernel" if staged else "ep_combine_kernel"]
     per_step = {n: sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for ev in marks) for i, n in enumerate(names)}
     kernel_us = {n: sum(v) / len(v) for n, v in per_step.items()}

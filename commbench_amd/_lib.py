@@ -20,6 +20,7 @@ SIGNATURES = {
     "mi_ep_workspace_status": (_int, [_vp, _vp]),
     "mi_ep_set_wait_limit": (_int, [ctypes.c_uint]),
     "mi_ep_set_dispatch_schedule": (_int, [_int]),
+    "mi_ep_dispatch_schedule_for": (_int, [_int, _int, _int, _int]),
     "mi_ep_dispatch_layout": (_int, [_vp, _int, _int, _int, _int, _int, _int,
                                      _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _size, _vp]),
     "mi_ep_route_order_bytes": (_size, [_int, _int]),

@@ -100,6 +100,18 @@ int mi_ep_set_dispatch_schedule(int schedule) {
   return MI_EP_OK;
 }
 
+int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, int row_bytes) {
+  if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK || num_experts <= 0 ||
+      num_experts > MI_EP_MAX_EXPERTS || row_bytes <= 0 || row_bytes % 16 != 0)
+    return MI_EP_EINVAL;
+  PermuteArgs a{};
+  a.num_tokens = num_tokens;
+  a.num_topk = num_topk;
+  a.num_experts = num_experts;
+  a.row_vecs = row_bytes / 16;
+  return destination_order_pays(a) ? kPermuteByDestination : kPermuteByToken;
+}
+
 size_t mi_ep_route_order_bytes(int num_tokens, int num_topk) {
   if (num_tokens <= 0 || num_topk <= 0) return 0;
   return static_cast<size_t>(num_tiles_for(num_tokens)) * kTileTokens * num_topk * 4 * sizeof(int);

@@ -94,6 +94,8 @@ constexpr int kPermuteAuto = 0;
 constexpr int kPermuteByToken = 1;        // wave per (token, 1 KiB): source read once, rows scattered
 constexpr int kPermuteByDestination = 2;  // needs route_order: rows written in destination order
 hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream);
+// The shape rule behind kPermuteAuto (reads num_tokens, num_topk, num_experts, row_vecs only).
+bool destination_order_pays(const PermuteArgs& a);
 hipError_t launch_gather_rows(const vec16* x, const float* x_scales, const int* recv_src_map, int num_rows,
                               int num_tokens, int row_vecs, int num_scales, vec16* recv_x,
                               float* recv_scales, hipStream_t stream);

@@ -323,7 +323,7 @@ __global__ __launch_bounds__(256) void ep_write_yardstick_kernel(vec16* __restri
 // and a tile leaves an expert a run of adjacent rows long enough for the memory controllers to
 // notice.  Measured: 14 KiB rows in 112 KiB runs gain 13-16 %, 8 KiB rows in 128 KiB runs gain
 // nothing, 7 KiB rows in 56 KiB runs lose 8 %.
-static bool destination_order_pays(const PermuteArgs& a) {
+bool destination_order_pays(const PermuteArgs& a) {
   const int tiles = (a.num_tokens + kTileTokens - 1) / kTileTokens;
   const int rounds = (tiles + kDies - 1) / kDies;
   if (tiles * 8 < rounds * kDies * 7) return false;  // more than 1/8 of the die-rounds idle

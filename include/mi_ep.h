@@ -78,6 +78,9 @@ int mi_ep_set_wait_limit(unsigned int max_polls);
  * 0 = chosen by shape (default), 1 = by token (wave per token and KiB, rows scattered),
  * 2 = by destination whenever route_order is given.  Results are identical. */
 int mi_ep_set_dispatch_schedule(int schedule);
+/* The kernel the default picks for a shape when route_order is given: 1 or 2 as above
+ * (kernel symbols ep_permute_kernel and ep_permute_tiles_kernel), or MI_EP_EINVAL. */
+int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, int row_bytes);
 
 /*
  * Fused single-pass layout: everything the reference spreads over

@@ -47,6 +47,14 @@ def test_host_only_entry_points():
     assert lib.mi_ep_route_order_bytes(257, 3) == 2 * 256 * 3 * 16
     assert lib.mi_ep_route_order_bytes(0, 8) == 0
     assert lib.mi_ep_set_dispatch_schedule(7) == -22 and lib.mi_ep_set_dispatch_schedule(0) == 0
+    # destination order: long rows, enough tiles for all eight dies, long enough runs per expert
+    assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 14336) == 2
+    assert lib.mi_ep_dispatch_schedule_for(4096, 8, 256, 14336) == 2
+    assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 7168) == 1      # 7 KiB rows
+    assert lib.mi_ep_dispatch_schedule_for(1024, 8, 256, 14336) == 1     # 4 tiles for 8 dies
+    assert lib.mi_ep_dispatch_schedule_for(8192, 2, 1024, 14336) == 1    # runs of 7 KiB per expert
+    assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 16384) == 1     # a tile's rows exceed L2
+    assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 100) == -22
     assert lib.mi_ep_workspace_bytes(8192, 8, 256, 9) == 0       # more than 8 ranks
     assert lib.mi_ep_workspace_bytes(8192, 9, 256, 8) == 0       # more than 8 slots
     assert lib.mi_ep_workspace_bytes(8192, 8, 250, 8) == 0       # experts not divisible by ranks
