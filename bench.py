@@ -34,6 +34,8 @@ def parse_args():
                          "(3 or more keeps the source out of the 256 MB memory-side cache)")
     ap.add_argument("--no-cold-source", action="store_true",
                     help="skip the extra pass with the source rows cycling through three buffers")
+    ap.add_argument("--no-host-path", action="store_true",
+                    help="skip the PCIe-inclusive pass through the host-pointer entry points")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short runs of the other configurations reported under other_configs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -127,6 +129,30 @@ class Workload:
         self.layout()
         self.dispatch()
         self.combine()
+
+
+def host_path(cfg, sample_tokens=2048):
+    """The same step through the host-pointer entry points (numpy in, numpy out) on a bounded
+    token sample: what a caller pays when the data lives in host memory.  Never `value`."""
+    import numpy as np
+    from commbench_amd import ops, workloads as wl
+    topk_np, w_np = wl.make_routing(cfg)
+    n = min(sample_tokens, cfg.num_tokens)
+    topk_np, w_np = topk_np[:n], w_np[:n]
+    rng = np.random.default_rng(wl.SEED_BASE + cfg.config_id)
+    x = rng.integers(0, 1 << 16, size=(n, cfg.row_bytes // 2), dtype=np.uint16)
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        d = ops.host_dispatch(x, None, topk_np, w_np, cfg.num_experts, cfg.num_ranks)
+        y = d["recv_x"] if cfg.payload == "bf16" else np.zeros((d["recv_x"].shape[0], cfg.hidden), np.uint16)
+        ops.host_combine(y, d["slot_map"], w_np)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    moved = x.nbytes + d["recv_x"].nbytes + y.nbytes + n * cfg.hidden * 2
+    return {"tokens_per_s": n / best, "ms": best * 1e3, "sample_tokens": n, "pcie_bytes": int(moved),
+            "note": "layout + dispatch + combine through mi_ep_host_*: pageable host arrays, device "
+                    "buffers allocated per call, best of 3"}
 
 
 def cpu_baseline(cfg, seconds):
@@ -381,6 +407,8 @@ def main():
             del owk
             torch.cuda.empty_cache()
         result["other_configs"] = others
+    if not args.no_host_path:
+        result["host_path"] = host_path(cfg)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
     print(json.dumps(result))

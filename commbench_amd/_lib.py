@@ -26,9 +26,13 @@ SIGNATURES = {
     "mi_ep_route_order_bytes": (_size, [_int, _int]),
     "mi_ep_dispatch": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int,
                               _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
-    "mi_ep_dispatch_cached": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp]),
+    "mi_ep_dispatch_cached": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _int, _vp]),
     "mi_ep_pull_indices": (_int, [_vp, _int, _int, _vp, _vp]),
     "mi_ep_combine": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp]),
+    "mi_ep_host_get_dispatch_layout": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int]),
+    "mi_ep_host_dispatch": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _int,
+                                   _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int]),
+    "mi_ep_host_combine": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
     "mi_ep_copy_yardstick": (_int, [_vp, _vp, _size, _vp]),
     "mi_ep_read_yardstick": (_int, [_vp, _size, _vp, _vp]),
     "mi_ep_write_yardstick": (_int, [_vp, _size, _vp]),

@@ -5,7 +5,7 @@ import subprocess
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libmi_ep.so")
-SOURCES = ["ep_abi.hip", "ep_layout.hip", "ep_permute.hip", "ep_combine.hip"]
+SOURCES = ["ep_abi.hip", "ep_host.hip", "ep_layout.hip", "ep_permute.hip", "ep_combine.hip"]
 
 # Packed fp32 instructions are switched off for every device compile of this tree.
 HIPCC_FLAGS = [

@@ -238,7 +238,8 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
 
 int mi_ep_dispatch_cached(const void* x, const float* x_scales, const int* recv_src_map,
                           int num_rows, int num_tokens, int row_bytes, int num_scales,
-                          void* recv_x, float* recv_scales, void* stream) {
+                          void* recv_x, float* recv_scales, int* ready_counters,
+                          int rows_per_counter, void* stream) {
   if (num_rows < 0 || num_tokens < 0 || row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0)
     return MI_EP_EINVAL;
   if (!aligned16(x) || !aligned16(recv_x)) return MI_EP_EINVAL;
@@ -246,9 +247,10 @@ int mi_ep_dispatch_cached(const void* x, const float* x_scales, const int* recv_
   if (num_rows > 0 && num_tokens > 0 && x == nullptr) return MI_EP_EINVAL;
   if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
   if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
+  if (ready_counters != nullptr && rows_per_counter <= 0) return MI_EP_EINVAL;
   return status_of(launch_gather_rows(static_cast<const vec16*>(x), x_scales, recv_src_map, num_rows,
                                       num_tokens, row_bytes / 16, num_scales, static_cast<vec16*>(recv_x),
-                                      recv_scales, as_stream(stream)));
+                                      recv_scales, ready_counters, rows_per_counter, as_stream(stream)));
 }
 
 int mi_ep_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_source_rank,

@@ -98,7 +98,8 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
 bool destination_order_pays(const PermuteArgs& a);
 hipError_t launch_gather_rows(const vec16* x, const float* x_scales, const int* recv_src_map, int num_rows,
                               int num_tokens, int row_vecs, int num_scales, vec16* recv_x,
-                              float* recv_scales, hipStream_t stream);
+                              float* recv_scales, int* ready_counters, int rows_per_counter,
+                              hipStream_t stream);
 hipError_t launch_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_source_rank,
                                int* pull_indices, hipStream_t stream);
 hipError_t launch_pad_rows(const PermuteArgs& a, hipStream_t stream);

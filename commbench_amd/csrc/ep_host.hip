@@ -1,0 +1,186 @@
+// Host-pointer twins of the device entry points: every pointer is ordinary host memory.
+// Each call allocates device buffers, copies the inputs over, runs the same kernels through
+// the device entry points, copies the outputs back and synchronises.  They are a convenience
+// for callers without a device-side pipeline (a harness that holds numpy arrays, a first
+// integration step); the transfers dominate, so nothing here is a measured path.
+#include "../../include/mi_ep.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace {
+
+// Device buffers that free themselves; `ok` turns false on the first failed allocation or copy.
+struct Staging {
+  hipError_t err = hipSuccess;
+  void* owned[24];
+  int count = 0;
+
+  ~Staging() {
+    for (int i = 0; i < count; ++i) (void)hipFree(owned[i]);
+  }
+  bool ok() const { return err == hipSuccess; }
+
+  template <typename T>
+  T* alloc(size_t n) {
+    if (!ok()) return nullptr;
+    if (count == static_cast<int>(sizeof(owned) / sizeof(owned[0]))) {
+      err = hipErrorOutOfMemory;
+      return nullptr;
+    }
+    void* p = nullptr;
+    err = hipMalloc(&p, (n > 0 ? n : 1) * sizeof(T) + 16);
+    if (err != hipSuccess) return nullptr;
+    owned[count++] = p;
+    return static_cast<T*>(p);
+  }
+  template <typename T>
+  T* upload(const T* host, size_t n) {
+    if (host == nullptr) return nullptr;
+    T* d = alloc<T>(n);
+    if (ok() && n > 0) err = hipMemcpy(d, host, n * sizeof(T), hipMemcpyHostToDevice);
+    return d;
+  }
+  template <typename T>
+  void download(T* host, const T* dev, size_t n) {
+    if (ok() && host != nullptr && n > 0) err = hipMemcpy(host, dev, n * sizeof(T), hipMemcpyDeviceToHost);
+  }
+  int status(int code) const {
+    if (code != MI_EP_OK) return code;
+    return err == hipSuccess ? MI_EP_OK : static_cast<int>(err);
+  }
+};
+
+int sync_status(int code) {
+  if (code != MI_EP_OK) return code;
+  const hipError_t e = hipStreamSynchronize(nullptr);
+  return e == hipSuccess ? MI_EP_OK : static_cast<int>(e);
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_ep_host_get_dispatch_layout(const int64_t* topk_idx, int* num_tokens_per_rank,
+                                   int* num_tokens_per_rdma_rank, int* num_tokens_per_expert,
+                                   bool* is_token_in_rank, int num_tokens, int num_topk, int num_ranks,
+                                   int num_experts) {
+  (void)num_tokens_per_rdma_rank;
+  if (num_tokens < 0 || num_topk <= 0 || num_ranks <= 0 || num_experts <= 0) return MI_EP_EINVAL;
+  if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
+  if (num_tokens > 0 && (topk_idx == nullptr || is_token_in_rank == nullptr)) return MI_EP_EINVAL;
+  Staging s;
+  const size_t tk = static_cast<size_t>(num_tokens) * num_topk;
+  const size_t tr = static_cast<size_t>(num_tokens) * num_ranks;
+  const int64_t* d_topk = s.upload(topk_idx, tk);
+  int* d_rank = s.alloc<int>(num_ranks);
+  int* d_expert = s.alloc<int>(num_experts);
+  bool* d_flags = s.alloc<bool>(tr);
+  if (!s.ok()) return s.status(MI_EP_OK);
+  int code = mi_ep_get_dispatch_layout(d_topk, d_rank, nullptr, d_expert, d_flags, num_tokens, num_topk,
+                                       num_ranks, num_experts, nullptr);
+  code = sync_status(code);
+  if (code != MI_EP_OK) return code;
+  s.download(num_tokens_per_rank, d_rank, num_ranks);
+  s.download(num_tokens_per_expert, d_expert, num_experts);
+  s.download(is_token_in_rank, d_flags, tr);
+  return s.status(MI_EP_OK);
+}
+
+int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
+                        const float* topk_weights, int num_tokens, int num_topk, int num_ranks,
+                        int num_experts, int expert_alignment, int row_bytes, int num_scales,
+                        int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
+                        int* expert_offsets, void* recv_x, float* recv_scales, int* recv_src_map,
+                        int64_t* recv_topk_idx, float* recv_topk_weights, int* slot_map,
+                        int capacity_rows) {
+  if (num_tokens < 0 || num_topk <= 0 || num_ranks <= 0 || num_experts <= 0 || expert_alignment < 1)
+    return MI_EP_EINVAL;
+  if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
+  if (expert_offsets == nullptr || recv_src_map == nullptr || slot_map == nullptr) return MI_EP_EINVAL;
+  if (num_tokens > 0 && (x == nullptr || topk_idx == nullptr)) return MI_EP_EINVAL;
+  if (capacity_rows > 0 && recv_x == nullptr) return MI_EP_EINVAL;
+  if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
+  if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
+  const size_t workspace_bytes = mi_ep_workspace_bytes(num_tokens > 0 ? num_tokens : 1, num_topk, num_experts, num_ranks);
+  if (workspace_bytes == 0) return MI_EP_EINVAL;
+
+  Staging s;
+  const size_t tk = static_cast<size_t>(num_tokens) * num_topk;
+  const size_t tr = static_cast<size_t>(num_tokens) * num_ranks;
+  const size_t cap = static_cast<size_t>(capacity_rows);
+  const unsigned char* d_x = s.upload(static_cast<const unsigned char*>(x), static_cast<size_t>(num_tokens) * row_bytes);
+  const float* d_scales = num_scales > 0 ? s.upload(x_scales, static_cast<size_t>(num_tokens) * num_scales) : nullptr;
+  const int64_t* d_topk = s.upload(topk_idx, tk);
+  const float* d_w = s.upload(topk_weights, tk);
+  int* d_rank = s.alloc<int>(num_ranks);
+  int* d_expert = s.alloc<int>(num_experts);
+  bool* d_flags = s.alloc<bool>(tr);
+  int* d_off = s.alloc<int>(static_cast<size_t>(num_experts) + 1);
+  int* d_slot_rel = s.alloc<int>(tk);
+  int* d_order = s.alloc<int>(mi_ep_route_order_bytes(num_tokens, num_topk) / sizeof(int));
+  unsigned char* d_ws = s.alloc<unsigned char>(workspace_bytes);
+  unsigned char* d_recv_x = s.alloc<unsigned char>(cap * row_bytes);
+  float* d_recv_scales = num_scales > 0 ? s.alloc<float>(cap * num_scales) : nullptr;
+  int* d_src_map = s.alloc<int>(cap);
+  int64_t* d_recv_idx = s.alloc<int64_t>(cap);
+  float* d_recv_w = s.alloc<float>(cap);
+  int* d_slot_map = s.alloc<int>(tk);
+  if (!s.ok()) return s.status(MI_EP_OK);
+
+  int code = mi_ep_workspace_init(d_ws, workspace_bytes, nullptr);
+  if (code == MI_EP_OK)
+    code = mi_ep_dispatch_layout(d_topk, num_tokens, num_topk, num_ranks, num_experts, expert_alignment, 0,
+                                 d_rank, d_expert, d_flags, d_off, nullptr, nullptr, d_slot_rel, nullptr, 0,
+                                 d_order, d_ws, workspace_bytes, nullptr);
+  if (code == MI_EP_OK)
+    code = mi_ep_dispatch(d_x, d_scales, d_topk, d_w, d_off, d_slot_rel, d_order, d_expert, num_tokens,
+                          num_topk, num_experts, expert_alignment, row_bytes, num_scales, d_recv_x,
+                          d_recv_scales, d_src_map, d_recv_idx, d_recv_w, d_slot_map, capacity_rows, nullptr);
+  if (code == MI_EP_OK) code = mi_ep_workspace_status(d_ws, nullptr);  // synchronises
+  if (code != MI_EP_OK) return code;
+
+  int total = 0;
+  s.download(&total, d_off + num_experts, 1);
+  if (!s.ok()) return s.status(MI_EP_OK);
+  const size_t rows = static_cast<size_t>(total) < cap ? static_cast<size_t>(total) : cap;
+  s.download(num_tokens_per_rank, d_rank, num_ranks);
+  s.download(num_tokens_per_expert, d_expert, num_experts);
+  s.download(is_token_in_rank, d_flags, tr);
+  s.download(expert_offsets, d_off, static_cast<size_t>(num_experts) + 1);
+  s.download(static_cast<unsigned char*>(recv_x), d_recv_x, rows * row_bytes);
+  if (num_scales > 0) s.download(recv_scales, d_recv_scales, rows * num_scales);
+  s.download(recv_src_map, d_src_map, rows);
+  s.download(recv_topk_idx, d_recv_idx, rows);
+  s.download(recv_topk_weights, d_recv_w, rows);
+  s.download(slot_map, d_slot_map, tk);
+  return s.status(MI_EP_OK);
+}
+
+int mi_ep_host_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
+                       const void* bias_0, const void* bias_1, int num_tokens, int num_topk, int hidden,
+                       void* combined_x) {
+  if (num_tokens < 0 || num_topk <= 0 || hidden <= 0 || hidden % 8 != 0 || num_rows < 0) return MI_EP_EINVAL;
+  if (num_rows > 0 && y == nullptr) return MI_EP_EINVAL;
+  if (num_tokens > 0 && (slot_map == nullptr || combined_x == nullptr)) return MI_EP_EINVAL;
+  Staging s;
+  const size_t tk = static_cast<size_t>(num_tokens) * num_topk;
+  const size_t th = static_cast<size_t>(num_tokens) * hidden;
+  const uint16_t* d_y = s.upload(static_cast<const uint16_t*>(y), static_cast<size_t>(num_rows) * hidden);
+  const int* d_map = s.upload(slot_map, tk);
+  const float* d_w = s.upload(topk_weights, tk);
+  const uint16_t* d_b0 = s.upload(static_cast<const uint16_t*>(bias_0), th);
+  const uint16_t* d_b1 = s.upload(static_cast<const uint16_t*>(bias_1), th);
+  uint16_t* d_out = s.alloc<uint16_t>(th);
+  if (!s.ok()) return s.status(MI_EP_OK);
+  int code = mi_ep_combine(d_y, num_rows, d_map, d_w, d_b0, d_b1, nullptr, num_tokens, num_topk, hidden,
+                           d_out, nullptr, nullptr);
+  code = sync_status(code);
+  if (code != MI_EP_OK) return code;
+  s.download(static_cast<uint16_t*>(combined_x), d_out, th);
+  return s.status(MI_EP_OK);
+}
+
+}  // extern "C"

@@ -255,6 +255,35 @@ __global__ __launch_bounds__(kPermuteThreads) void ep_gather_rows_kernel(
           live ? x_scales[static_cast<size_t>(token) * num_scales + j] : 0.0f;
 }
 
+// The same pull with arrival counters: one workgroup per destination row; when the whole row
+// (pads included) is in place, ready_counters[row / rows_per_counter] is bumped once, with
+// release semantics, so that a consumer that sees a block's counter reach its row count may
+// read the block (the per-128-row barrier of the reference's pull dispatch,
+// example056 .cu:181-202).
+__global__ __launch_bounds__(kPermuteThreads) void ep_gather_rows_ready_kernel(
+    const vec16* __restrict__ x, const float* __restrict__ x_scales, const int* __restrict__ recv_src_map,
+    const int num_tokens, const int row_vecs, const int num_scales, vec16* __restrict__ recv_x,
+    float* __restrict__ recv_scales, int* __restrict__ ready_counters, const int rows_per_counter) {
+  const int row = static_cast<int>(blockIdx.x);
+  const int tid = static_cast<int>(threadIdx.x);
+  const int token = recv_src_map[row];
+  const bool live = token >= 0 && token < num_tokens;
+  const vec16* src = x + static_cast<size_t>(live ? token : 0) * row_vecs;
+  vec16* dst = recv_x + static_cast<size_t>(row) * row_vecs;
+  const vec16 zero = {0u, 0u, 0u, 0u};
+  for (int v = tid; v < row_vecs; v += kPermuteThreads)
+    __builtin_nontemporal_store(live ? src[v] : zero, dst + v);
+  if (recv_scales != nullptr)
+    for (int j = tid; j < num_scales; j += kPermuteThreads)
+      recv_scales[static_cast<size_t>(row) * num_scales + j] =
+          live ? x_scales[static_cast<size_t>(token) * num_scales + j] : 0.0f;
+  __threadfence();  // every thread's stores are visible device-wide before the barrier
+  __syncthreads();
+  if (tid == 0)
+    __hip_atomic_fetch_add(&ready_counters[row / rows_per_counter], 1, __ATOMIC_RELEASE,
+                           __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __global__ __launch_bounds__(256) void ep_pull_indices_kernel(const int* __restrict__ recv_src_map,
                                                              const int num_rows,
                                                              const int tokens_per_source_rank,
@@ -364,8 +393,15 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
 
 hipError_t launch_gather_rows(const vec16* x, const float* x_scales, const int* recv_src_map, int num_rows,
                               int num_tokens, int row_vecs, int num_scales, vec16* recv_x,
-                              float* recv_scales, hipStream_t stream) {
+                              float* recv_scales, int* ready_counters, int rows_per_counter,
+                              hipStream_t stream) {
   if (num_rows == 0) return hipSuccess;
+  if (ready_counters != nullptr) {
+    hipLaunchKernelGGL(ep_gather_rows_ready_kernel, dim3(static_cast<unsigned>(num_rows)),
+                       dim3(kPermuteThreads), 0, stream, x, x_scales, recv_src_map, num_tokens, row_vecs,
+                       num_scales, recv_x, recv_scales, ready_counters, rows_per_counter);
+    return hipGetLastError();
+  }
   const int batch_vecs = row_vecs > kWave ? 2 : 1;
   const int per_batch = batch_vecs * kWave;
   const int batches = (row_vecs + per_batch - 1) / per_batch;

@@ -268,9 +268,12 @@ def dispatch(x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Te
 
 
 def dispatch_cached(x: torch.Tensor, scales: Optional[torch.Tensor], recv_src_map: torch.Tensor,
-                    num_rows: Optional[int] = None):
+                    num_rows: Optional[int] = None, ready_counters: Optional[torch.Tensor] = None,
+                    rows_per_counter: int = 128):
     """Pull-mode dispatch of a new payload with the source map of an earlier dispatch (the
-    reference's cached mode).  Returns (recv_x, recv_scales); pad rows are zero."""
+    reference's cached mode).  Returns (recv_x, recv_scales); pad rows are zero.  With
+    `ready_counters` (zeroed int32[ceil(rows / rows_per_counter)]) every row bumps its block's
+    counter once it is in place, as the ThunderKittens example's pull dispatch does."""
     _require(x.is_cuda and x.dim() == 2 and x.is_contiguous(), "x must be a contiguous 2-D GPU tensor")
     _require(recv_src_map.dtype == torch.int32 and recv_src_map.dim() == 1 and recv_src_map.is_contiguous(),
              "recv_src_map must be contiguous int32 [rows]")
@@ -286,10 +289,16 @@ def dispatch_cached(x: torch.Tensor, scales: Optional[torch.Tensor], recv_src_ma
     recv_x = torch.empty((rows, x.shape[1]), dtype=x.dtype, device=x.device)
     recv_scales = (torch.empty((rows, num_scales), dtype=torch.float32, device=x.device)
                    if scales is not None else None)
+    if ready_counters is not None:
+        _require(ready_counters.is_cuda and ready_counters.dtype == torch.int32
+                 and ready_counters.is_contiguous() and rows_per_counter > 0
+                 and ready_counters.numel() * rows_per_counter >= rows,
+                 "ready_counters must be contiguous int32 [ceil(rows / rows_per_counter)]")
     lib = _lib.load()
     _lib.check(lib.mi_ep_dispatch_cached(_ptr(x), _ptr(scales), _ptr(recv_src_map), rows, x.shape[0],
                                          row_bytes, num_scales, _ptr(recv_x), _ptr(recv_scales),
-                                         _stream()), "mi_ep_dispatch_cached")
+                                         _ptr(ready_counters), rows_per_counter, _stream()),
+               "mi_ep_dispatch_cached")
     return recv_x, recv_scales
 
 
@@ -315,3 +324,89 @@ def copy_yardstick(dst: torch.Tensor, src: torch.Tensor) -> None:
     lib = _lib.load()
     _lib.check(lib.mi_ep_copy_yardstick(_ptr(dst), _ptr(src), nbytes, _stream()),
                "mi_ep_copy_yardstick")
+
+
+# ---- host-pointer twins: numpy in, numpy out (transfers included; never a measured path) -------
+
+def _np(a, dtype):
+    import numpy as np
+    if a is None:
+        return None
+    a = np.ascontiguousarray(a)
+    _require(a.dtype == np.dtype(dtype), f"expected a {np.dtype(dtype).name} array")
+    return a
+
+
+def _np_ptr(a):
+    return None if a is None else a.ctypes.data
+
+
+def host_get_dispatch_layout(topk_idx, num_experts: int, num_ranks: int):
+    """get_dispatch_layout on host arrays: (num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank)."""
+    import numpy as np
+    topk_idx = _np(topk_idx, np.int64)
+    _require(topk_idx.ndim == 2, "topk_idx must be [num_tokens, num_topk]")
+    T, K = topk_idx.shape
+    per_rank = np.empty(num_ranks, dtype=np.int32)
+    per_expert = np.empty(num_experts, dtype=np.int32)
+    flags = np.empty((T, num_ranks), dtype=np.bool_)
+    _lib.check(_lib.load().mi_ep_host_get_dispatch_layout(
+        _np_ptr(topk_idx), _np_ptr(per_rank), None, _np_ptr(per_expert), _np_ptr(flags), T, K, num_ranks,
+        num_experts), "mi_ep_host_get_dispatch_layout")
+    return per_rank, per_expert, flags
+
+
+def host_dispatch(x, scales, topk_idx, topk_weights, num_experts: int, num_ranks: int,
+                  expert_alignment: int = 1):
+    """Layout + dispatch on host arrays.  `x` is a [num_tokens, row] array of any 1-, 2- or 4-byte
+    dtype; returns a dict with the layout outputs, expert_offsets, slot_map and the recv_* arrays
+    trimmed to expert_offsets[-1] rows."""
+    import numpy as np
+    topk_idx = _np(topk_idx, np.int64)
+    T, K = topk_idx.shape
+    x = np.ascontiguousarray(x)
+    _require(x.ndim == 2 and x.shape[0] == T, "x must be [num_tokens, row]")
+    row_bytes = x.shape[1] * x.itemsize
+    scales = _np(scales, np.float32)
+    topk_weights = _np(topk_weights, np.float32)
+    S = 0 if scales is None else scales.shape[1]
+    cap = T * K + num_experts * (expert_alignment - 1)
+    out = dict(
+        num_tokens_per_rank=np.empty(num_ranks, dtype=np.int32),
+        num_tokens_per_expert=np.empty(num_experts, dtype=np.int32),
+        is_token_in_rank=np.empty((T, num_ranks), dtype=np.bool_),
+        expert_offsets=np.empty(num_experts + 1, dtype=np.int32),
+        recv_x=np.empty((cap, x.shape[1]), dtype=x.dtype),
+        recv_scales=None if scales is None else np.empty((cap, S), dtype=np.float32),
+        recv_src_map=np.empty(cap, dtype=np.int32),
+        recv_topk_idx=np.empty(cap, dtype=np.int64),
+        recv_topk_weights=np.empty(cap, dtype=np.float32),
+        slot_map=np.empty((T, K), dtype=np.int32))
+    _lib.check(_lib.load().mi_ep_host_dispatch(
+        _np_ptr(x), _np_ptr(scales), _np_ptr(topk_idx), _np_ptr(topk_weights), T, K, num_ranks, num_experts,
+        expert_alignment, row_bytes, S, _np_ptr(out["num_tokens_per_rank"]),
+        _np_ptr(out["num_tokens_per_expert"]), _np_ptr(out["is_token_in_rank"]),
+        _np_ptr(out["expert_offsets"]), _np_ptr(out["recv_x"]), _np_ptr(out["recv_scales"]),
+        _np_ptr(out["recv_src_map"]), _np_ptr(out["recv_topk_idx"]), _np_ptr(out["recv_topk_weights"]),
+        _np_ptr(out["slot_map"]), cap), "mi_ep_host_dispatch")
+    rows = int(out["expert_offsets"][-1])
+    for key in ("recv_x", "recv_scales", "recv_src_map", "recv_topk_idx", "recv_topk_weights"):
+        if out[key] is not None:
+            out[key] = out[key][:rows]
+    return out
+
+
+def host_combine(y_bits, slot_map, topk_weights=None, bias_0=None, bias_1=None):
+    """combine on host arrays of bf16 bit patterns (uint16): returns uint16 [num_tokens, hidden]."""
+    import numpy as np
+    y_bits = _np(y_bits, np.uint16)
+    slot_map = _np(slot_map, np.int32)
+    T, K = slot_map.shape
+    H = y_bits.shape[1]
+    topk_weights = _np(topk_weights, np.float32)
+    bias_0, bias_1 = _np(bias_0, np.uint16), _np(bias_1, np.uint16)
+    out = np.empty((T, H), dtype=np.uint16)
+    _lib.check(_lib.load().mi_ep_host_combine(
+        _np_ptr(y_bits), y_bits.shape[0], _np_ptr(slot_map), _np_ptr(topk_weights), _np_ptr(bias_0),
+        _np_ptr(bias_1), T, K, H, _np_ptr(out)), "mi_ep_host_combine")
+    return out

@@ -165,10 +165,16 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
  * recv_x / recv_scales becomes a byte copy of token recv_src_map[i]; rows whose map entry is
  * negative (pads) or not below num_tokens are zero-filled.  No routing tables are read.
  * Same size and alignment rules as mi_ep_dispatch.
+ *   ready_counters  NULL, or int32[ceil(num_rows / rows_per_counter)] that the caller has zeroed:
+ *                   counter i is incremented once (device-scope release) for every row of block
+ *                   i, pads included, after the row is in place; a consumer on another stream
+ *                   may read block i once the counter equals the block's row count.  This is the
+ *                   per-row-block arrival barrier of the same example (:196-202, ROW_BLOCK = 128).
  */
 int mi_ep_dispatch_cached(const void* x, const float* x_scales, const int* recv_src_map,
                           int num_rows, int num_tokens, int row_bytes, int num_scales,
-                          void* recv_x, float* recv_scales, void* stream);
+                          void* recv_x, float* recv_scales, int* ready_counters,
+                          int rows_per_counter, void* stream);
 
 /*
  * The same map in the ThunderKittens example's format
@@ -198,6 +204,35 @@ int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float*
                   const void* bias_0, const void* bias_1, const float* recv_topk_weights,
                   int num_tokens, int num_topk, int hidden, void* combined_x,
                   float* combined_topk_weights, void* stream);
+
+/*
+ * Host-pointer twins: the same operations with every pointer in ordinary host memory.  Each call
+ * allocates device buffers, copies inputs over, runs the kernels above on the null stream, copies
+ * the outputs back and returns after synchronising; errors as above.  They serve callers without a
+ * device-side pipeline (the reference's harnesses keep their data in host vectors between
+ * hipMemcpy calls, example042 .cu:243-293); transfers dominate their time.
+ *   mi_ep_host_get_dispatch_layout  twin of mi_ep_get_dispatch_layout
+ *   mi_ep_host_dispatch             layout + dispatch in one call: the layout outputs
+ *                                   (num_tokens_per_rank / _expert, is_token_in_rank, any of them
+ *                                   may be NULL) and expert_offsets come back with the permuted
+ *                                   rows; only the first min(expert_offsets[E], capacity_rows)
+ *                                   rows of the recv_* arrays are written
+ *   mi_ep_host_combine              twin of mi_ep_combine (without the travelled weights)
+ */
+int mi_ep_host_get_dispatch_layout(const int64_t* topk_idx, int* num_tokens_per_rank,
+                                   int* num_tokens_per_rdma_rank, int* num_tokens_per_expert,
+                                   bool* is_token_in_rank, int num_tokens, int num_topk, int num_ranks,
+                                   int num_experts);
+int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
+                        const float* topk_weights, int num_tokens, int num_topk, int num_ranks,
+                        int num_experts, int expert_alignment, int row_bytes, int num_scales,
+                        int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
+                        int* expert_offsets, void* recv_x, float* recv_scales, int* recv_src_map,
+                        int64_t* recv_topk_idx, float* recv_topk_weights, int* slot_map,
+                        int capacity_rows);
+int mi_ep_host_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
+                       const void* bias_0, const void* bias_1, int num_tokens, int num_topk, int hidden,
+                       void* combined_x);
 
 /*
  * 16-byte streaming copy used as the measured HBM ceiling next to the nominal

@@ -277,6 +277,15 @@ def test_cached_pull_dispatch_and_pull_indices(oracle, payload):
     np.testing.assert_array_equal(gu.as_bytes(got_x), want_x)
     if s2 is not None:
         np.testing.assert_array_equal(got_s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+    # the same pull with arrival counters: same rows, every 128-row block counted in full
+    ready = torch.zeros((rows + 127) // 128, dtype=torch.int32, device=gu.DEV)
+    got_x2, got_s2 = ops.dispatch_cached(x2.to(gu.DEV), None if s2 is None else s2.to(gu.DEV),
+                                         h.recv_src_map, num_rows=rows, ready_counters=ready)
+    np.testing.assert_array_equal(gu.as_bytes(got_x2), want_x)
+    if s2 is not None:
+        np.testing.assert_array_equal(got_s2.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+    want_ready = np.minimum(128, rows - 128 * np.arange(ready.numel())).astype(np.int32)
+    np.testing.assert_array_equal(ready.cpu().numpy(), want_ready)
     # and with the first payload it is the first dispatch again
     again, _ = ops.dispatch_cached(x_cpu.to(gu.DEV), None if scales_cpu is None else scales_cpu.to(gu.DEV),
                                    h.recv_src_map, num_rows=rows)
