@@ -236,6 +236,65 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
   return status_of(e);
 }
 
+int mi_ep_dispatch_ranks(const void* x, const float* x_scales, const int64_t* topk_idx,
+                         const float* topk_weights, const int* rank_slot_idx, int rank_slot_base,
+                         const int* num_tokens_per_rank, const int* expand_slot_map, int num_tokens,
+                         int num_topk, int num_ranks, int num_experts, int row_bytes, int num_scales,
+                         int source_token_base, int local_expert_ids, void* recv_x, float* recv_scales,
+                         int64_t* recv_topk_idx, float* recv_topk_weights, int* recv_src_metadata,
+                         int* rank_row_map, int* combine_map, int* psum_rank_tokens, int capacity_rows,
+                         void* stream) {
+  if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
+  if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
+  if (num_tokens_per_rank == nullptr || psum_rank_tokens == nullptr) return MI_EP_EINVAL;
+  if (capacity_rows > 0 && recv_x == nullptr) return MI_EP_EINVAL;
+  if (!aligned16(x) || !aligned16(recv_x)) return MI_EP_EINVAL;
+  if (num_tokens > 0 &&
+      (x == nullptr || topk_idx == nullptr || rank_slot_idx == nullptr || rank_row_map == nullptr))
+    return MI_EP_EINVAL;
+  if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
+  if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
+
+  RankPermuteArgs a{};
+  a.x = static_cast<const vec16*>(x);
+  a.x_scales = x_scales;
+  a.topk_idx = topk_idx;
+  a.topk_weights = topk_weights;
+  a.rank_slot_idx = rank_slot_idx;
+  a.num_tokens_per_rank = num_tokens_per_rank;
+  a.expand_slot_map = expand_slot_map;
+  a.recv_x = static_cast<vec16*>(recv_x);
+  a.recv_scales = recv_scales;
+  a.recv_topk_idx = recv_topk_idx;
+  a.recv_topk_weights = recv_topk_weights;
+  a.recv_src_metadata = recv_src_metadata;
+  a.rank_row_map = rank_row_map;
+  a.combine_map = combine_map;
+  a.psum_rank_tokens = psum_rank_tokens;
+  a.num_tokens = num_tokens;
+  a.num_topk = num_topk;
+  a.num_ranks = num_ranks;
+  a.num_experts = num_experts;
+  a.experts_per_rank = num_experts / num_ranks;
+  a.row_vecs = row_bytes / 16;
+  a.num_scales = num_scales;
+  a.capacity_rows = capacity_rows;
+  a.rank_slot_base = rank_slot_base;
+  a.source_token_base = source_token_base;
+  a.local_expert_ids = local_expert_ids != 0;
+  return status_of(launch_permute_ranks(a, as_stream(stream)));
+}
+
+int mi_ep_combine_rank_weights(const float* recv_topk_weights, const int* rank_row_map, int num_tokens,
+                               int num_topk, int num_rows, float* combined_topk_weights, void* stream) {
+  if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK || num_rows < 0) return MI_EP_EINVAL;
+  if (static_cast<long long>(num_tokens) * num_topk >= (1LL << 30)) return MI_EP_EINVAL;
+  if (num_tokens > 0 && (rank_row_map == nullptr || combined_topk_weights == nullptr)) return MI_EP_EINVAL;
+  if (num_rows > 0 && recv_topk_weights == nullptr) return MI_EP_EINVAL;
+  return status_of(launch_gather_rank_weights(recv_topk_weights, rank_row_map, num_tokens, num_topk, num_rows,
+                                              combined_topk_weights, as_stream(stream)));
+}
+
 int mi_ep_dispatch_cached(const void* x, const float* x_scales, const int* recv_src_map,
                           int num_rows, int num_tokens, int row_bytes, int num_scales,
                           void* recv_x, float* recv_scales, int* ready_counters,

@@ -104,6 +104,40 @@ hipError_t launch_pull_indices(const int* recv_src_map, int num_rows, int tokens
                                int* pull_indices, hipStream_t stream);
 hipError_t launch_pad_rows(const PermuteArgs& a, hipStream_t stream);
 
+// Dispatch de-duplicated by destination rank: one row per (token, rank that owns one of its experts).
+struct RankPermuteArgs {
+  const vec16* x;
+  const float* x_scales;
+  const int64_t* topk_idx;
+  const float* topk_weights;
+  const int* rank_slot_idx;        // from the layout kernel: rank_slot_base + slot on first-of-rank slots
+  const int* num_tokens_per_rank;  // from the layout kernel
+  const int* expand_slot_map;      // rows of the expanded buffer, or null
+  vec16* recv_x;
+  float* recv_scales;
+  int64_t* recv_topk_idx;     // [rows, K]
+  float* recv_topk_weights;   // [rows, K]
+  int* recv_src_metadata;     // [rows, 2 + K]
+  int* rank_row_map;          // [T, K]
+  int* combine_map;           // [T, K] or null: each received row once
+  int* psum_rank_tokens;      // [R]
+  int num_tokens;
+  int num_topk;
+  int num_ranks;
+  int num_experts;
+  int experts_per_rank;
+  int row_vecs;
+  int num_scales;
+  int capacity_rows;
+  int rank_slot_base;
+  int source_token_base;
+  int local_expert_ids;
+};
+hipError_t launch_permute_ranks(const RankPermuteArgs& a, hipStream_t stream);
+hipError_t launch_gather_rank_weights(const float* recv_topk_weights, const int* rank_row_map, int num_tokens,
+                                      int num_topk, int num_rows, float* combined_topk_weights,
+                                      hipStream_t stream);
+
 // ---- combine ----------------------------------------------------------------
 struct CombineArgs {
   const vec16* y;

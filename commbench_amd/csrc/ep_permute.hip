@@ -194,6 +194,115 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
   }
 }
 
+// Dispatch de-duplicated by destination rank (the reference's own format: payload role of
+// dispatch_impl, example080 .cu:241-256, then the copy epilogue without expansion,
+// example081 .cu:22-60).  Same wave-per-(token, KiB) shape as ep_permute_kernel; a token's
+// destinations are the first slot of each distinct rank, whose position inside the rank's rows
+// the layout kernel has already fixed (rank_slot_idx).
+__global__ __launch_bounds__(kPushThreads) void ep_permute_ranks_kernel(const RankPermuteArgs a,
+                                                                       const int batches_per_row) {
+  const int lane = lane_id();
+  const int wave = static_cast<int>(threadIdx.x) >> 6;
+  const long long unit = static_cast<long long>(blockIdx.x) * kPushWaves + wave;
+  const int token = static_cast<int>(unit / batches_per_row);
+  const int batch = static_cast<int>(unit - static_cast<long long>(token) * batches_per_row);
+  if (unit == 0 && lane < a.num_ranks) {  // inclusive rows per rank, for callers that size by it
+    int run = 0;
+    for (int r = 0; r <= lane; ++r) run += a.num_tokens_per_rank[r];
+    a.psum_rank_tokens[lane] = run;
+  }
+  if (token >= a.num_tokens) return;
+  const int K = a.num_topk;
+
+  const vec16* src = a.x + static_cast<size_t>(token) * a.row_vecs;
+  const int v = batch * kWave + lane;
+  vec16 buf = {0u, 0u, 0u, 0u};
+  if (v < a.row_vecs) buf = src[v];
+
+  // Lane k < K resolves slot k: its rank, and on the first slot of a rank the row it opens.
+  const size_t i = static_cast<size_t>(token) * K + (lane < K ? lane : 0);
+  int64_t expert = -1;
+  int rank = -1, own_row = -1;
+  bool opens = false;
+  if (lane < K) {
+    expert = a.topk_idx[i];
+    if (expert >= 0 && expert < static_cast<int64_t>(a.num_experts)) {
+      rank = static_cast<int>(expert) / a.experts_per_rank;
+      const int slot = a.rank_slot_idx[i];
+      opens = slot >= 0;
+      if (opens) {
+        int base = 0;
+        for (int r = 0; r < rank; ++r) base += a.num_tokens_per_rank[r];
+        own_row = base + (slot - a.rank_slot_base);
+        if (own_row < 0 || own_row >= a.capacity_rows) own_row = -1;  // dropped
+      }
+    }
+  }
+
+  if (batch == 0) {
+    // The row that carries each route: the one its rank's first slot opened.
+    int route_row = -1;
+    for (int j = 0; j < K; ++j) {
+      const int rank_j = wave_read(rank, j);
+      const int row_j = wave_read(own_row, j);
+      const bool opens_j = wave_read(static_cast<int>(opens), j) != 0;
+      if (opens_j && rank >= 0 && rank == rank_j) route_row = row_j;
+    }
+    if (lane < K) {
+      a.rank_row_map[i] = route_row;
+      if (a.combine_map != nullptr) a.combine_map[i] = own_row;
+    }
+    const int stride = 2 + K;
+    for (int j = 0; j < K; ++j) {
+      const int row = wave_read(own_row, j);
+      if (row < 0) continue;
+      const int rank_j = wave_read(rank, j);
+      if (lane < K) {
+        const bool local = rank == rank_j;
+        const size_t o = static_cast<size_t>(row) * K + lane;
+        if (a.recv_topk_idx != nullptr)
+          a.recv_topk_idx[o] =
+              local ? expert - (a.local_expert_ids ? static_cast<int64_t>(rank_j) * a.experts_per_rank : 0) : -1;
+        if (a.recv_topk_weights != nullptr)
+          a.recv_topk_weights[o] = local ? (a.topk_weights != nullptr ? a.topk_weights[i] : 1.0f) : 0.0f;
+        if (a.recv_src_metadata != nullptr)
+          a.recv_src_metadata[static_cast<size_t>(row) * stride + 2 + lane] =
+              (local && a.expand_slot_map != nullptr) ? a.expand_slot_map[i] : -1;
+      }
+      if (lane == 0 && a.recv_src_metadata != nullptr) {
+        a.recv_src_metadata[static_cast<size_t>(row) * stride + 0] = a.source_token_base + token;
+        a.recv_src_metadata[static_cast<size_t>(row) * stride + 1] = rank_j;
+      }
+      if (a.recv_scales != nullptr)
+        for (int s = lane; s < a.num_scales; s += kWave)
+          a.recv_scales[static_cast<size_t>(row) * a.num_scales + s] =
+              a.x_scales[static_cast<size_t>(token) * a.num_scales + s];
+    }
+  }
+
+#pragma unroll
+  for (int j = 0; j < kMaxTopk; ++j) {
+    if (j < K) {
+      const int row = wave_read(own_row, j);
+      if (row >= 0 && v < a.row_vecs)
+        __builtin_nontemporal_store(buf, a.recv_x + static_cast<size_t>(row) * a.row_vecs + v);
+    }
+  }
+}
+
+// combined_topk_weights[t,k] = the weight that travelled with route (t,k) in the per-rank format.
+__global__ __launch_bounds__(256) void ep_gather_rank_weights_kernel(const float* __restrict__ recv_topk_weights,
+                                                                    const int* __restrict__ rank_row_map,
+                                                                    const int total, const int num_topk,
+                                                                    const int num_rows,
+                                                                    float* __restrict__ out) {
+  const int i = static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
+  if (i >= total) return;
+  const int row = rank_row_map[i];
+  const int k = i % num_topk;
+  out[i] = (row >= 0 && row < num_rows) ? recv_topk_weights[static_cast<size_t>(row) * num_topk + k] : 0.0f;
+}
+
 // Zero-fills the rows that expert_alignment > 1 leaves between a segment's last
 // route and the next segment.  One workgroup per expert.
 __global__ __launch_bounds__(kPermuteThreads) void ep_pad_rows_kernel(const PermuteArgs a) {
@@ -388,6 +497,28 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
   hipLaunchKernelGGL((ep_permute_kernel<1, true>), dim3(static_cast<unsigned>(blocks)), dim3(kPushThreads), 0,
                      stream, a, batches);
+  return hipGetLastError();
+}
+
+hipError_t launch_permute_ranks(const RankPermuteArgs& a, hipStream_t stream) {
+  const int batches = (a.row_vecs + kWave - 1) / kWave;
+  // At least one unit, so that the per-rank row totals are written for an empty batch too.
+  const long long units = a.num_tokens > 0 ? static_cast<long long>(a.num_tokens) * batches : 1;
+  const long long blocks = (units + kPushWaves - 1) / kPushWaves;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(ep_permute_ranks_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kPushThreads), 0, stream,
+                     a, batches);
+  return hipGetLastError();
+}
+
+hipError_t launch_gather_rank_weights(const float* recv_topk_weights, const int* rank_row_map, int num_tokens,
+                                      int num_topk, int num_rows, float* combined_topk_weights,
+                                      hipStream_t stream) {
+  const long long total = static_cast<long long>(num_tokens) * num_topk;
+  if (total == 0) return hipSuccess;
+  hipLaunchKernelGGL(ep_gather_rank_weights_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                     stream, recv_topk_weights, rank_row_map, static_cast<int>(total), num_topk, num_rows,
+                     combined_topk_weights);
   return hipGetLastError();
 }
 

@@ -168,7 +168,7 @@ class Buffer:
     def dispatch(self, x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Tensor,
                  topk_weights: Optional[torch.Tensor], expert_alignment: int = 1,
                  num_channels: int = 0, handle: Optional[DispatchHandle] = None,
-                 capacity_rows: Optional[int] = None):
+                 capacity_rows: Optional[int] = None, rank_slot_base: Optional[int] = None):
         """Layout (unless `handle` is given) + permute into the expert-contiguous buffer.
 
         Returns (recv_x, recv_scales, recv_src_map, handle).  Buffers hold `capacity_rows` rows
@@ -176,7 +176,7 @@ class Buffer:
         beyond handle.num_recv_rows() are unspecified.
         """
         if handle is None:
-            handle = self.dispatch_layout(topk_idx, expert_alignment, num_channels)
+            handle = self.dispatch_layout(topk_idx, expert_alignment, num_channels, rank_slot_base)
         T, K, E = handle.num_tokens, handle.num_topk, handle.num_experts
         _require(x.is_cuda and x.dim() == 2 and x.is_contiguous() and x.shape[0] == T,
                  "x must be a contiguous [num_tokens, hidden] GPU tensor")
@@ -209,6 +209,84 @@ class Buffer:
             _ptr(handle.recv_src_map), _ptr(handle.recv_topk_idx), _ptr(handle.recv_topk_weights),
             _ptr(handle.slot_map), capacity_rows, _stream()), "mi_ep_dispatch")
         return recv_x, recv_scales, handle.recv_src_map, handle
+
+
+@dataclass
+class RankDispatchHandle:
+    """What the per-rank dispatch hands to combine (the reference's handle, example082 bar.py:744-755)."""
+    layout: DispatchHandle
+    psum_rank_tokens: torch.Tensor        # int32[R], inclusive rows per rank
+    recv_src_metadata: torch.Tensor       # int32[capacity, 2 + K]
+    rank_row_map: torch.Tensor            # int32[T, K], row carrying each route
+    combine_map: torch.Tensor             # int32[T, K], each received row once
+    recv_scales: Optional[torch.Tensor] = None
+
+    def num_recv_rows(self) -> int:
+        """Rows received over all ranks; synchronises the stream."""
+        return int(self.psum_rank_tokens[-1].item())
+
+
+def dispatch_ranks(buffer: "Buffer", x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Tensor,
+                   topk_weights: Optional[torch.Tensor], num_max_tokens_per_rank: Optional[int] = None,
+                   rank_idx: int = 0, local_expert_ids: bool = False, expand: bool = False):
+    """The reference's dispatch in its own receive format: one row per (token, destination rank),
+    ranks' rows in token order (deterministic mode).  Returns (recv_x, recv_topk_idx,
+    recv_topk_weights, handle) as DeepEP's `buffer.dispatch` does (example080 bar.py:725);
+    `rank_idx * num_max_tokens_per_rank` offsets the source token ids in the metadata.
+    With `expand`, the expert-contiguous dispatch runs too and the metadata names its rows."""
+    T, K = _check_routing(topk_idx, buffer.num_experts, buffer.num_ranks)
+    E, R, dev = buffer.num_experts, buffer.num_ranks, topk_idx.device
+    max_tokens = T if num_max_tokens_per_rank is None else num_max_tokens_per_rank
+    base = rank_idx * max_tokens
+    if expand:
+        _, _, _, h = buffer.dispatch(x, scales, topk_idx, topk_weights, rank_slot_base=base)
+    else:
+        h = buffer.dispatch_layout(topk_idx, rank_slot_base=base, route_order=False)
+    _require(x.is_cuda and x.dim() == 2 and x.is_contiguous() and x.shape[0] == T,
+             "x must be a contiguous [num_tokens, hidden] GPU tensor")
+    row_bytes = x.shape[1] * x.element_size()
+    _require(row_bytes % 16 == 0, "row size must be a multiple of 16 bytes")
+    S = 0
+    if scales is not None:
+        _require(scales.dtype == torch.float32 and scales.dim() == 2 and scales.is_contiguous()
+                 and scales.shape[0] == T, "scales must be contiguous float32 [num_tokens, S]")
+        S = scales.shape[1]
+    cap = T * min(K, R)
+    recv_x = torch.empty((cap, x.shape[1]), dtype=x.dtype, device=dev)
+    recv_scales = torch.empty((cap, S), dtype=torch.float32, device=dev) if scales is not None else None
+    recv_idx = torch.empty((cap, K), dtype=torch.int64, device=dev)
+    recv_w = torch.empty((cap, K), dtype=torch.float32, device=dev)
+    rh = RankDispatchHandle(
+        layout=h, psum_rank_tokens=torch.empty(R, dtype=torch.int32, device=dev),
+        recv_src_metadata=torch.empty((cap, 2 + K), dtype=torch.int32, device=dev),
+        rank_row_map=torch.empty((T, K), dtype=torch.int32, device=dev),
+        combine_map=torch.empty((T, K), dtype=torch.int32, device=dev), recv_scales=recv_scales)
+    _lib.check(_lib.load().mi_ep_dispatch_ranks(
+        _ptr(x), _ptr(scales), _ptr(topk_idx), _ptr(topk_weights), _ptr(h.rank_slot_idx), base,
+        _ptr(h.num_tokens_per_rank), _ptr(h.slot_map) if expand else None, T, K, R, E, row_bytes, S, base,
+        1 if local_expert_ids else 0, _ptr(recv_x), _ptr(recv_scales), _ptr(recv_idx), _ptr(recv_w),
+        _ptr(rh.recv_src_metadata), _ptr(rh.rank_row_map), _ptr(rh.combine_map), _ptr(rh.psum_rank_tokens),
+        cap, _stream()), "mi_ep_dispatch_ranks")
+    return recv_x, recv_idx, recv_w, rh
+
+
+def combine_ranks(y: torch.Tensor, handle: RankDispatchHandle, recv_topk_weights: Optional[torch.Tensor] = None,
+                  bias=None):
+    """The reference's combine of the per-rank format: the ordered sum of the rows a token sent
+    out, one per rank (+ biases); with `recv_topk_weights` also the weights that travelled
+    (combined_topk_weights, example082 bar.py:757-765)."""
+    out = combine(y, handle.combine_map, None, bias)
+    if recv_topk_weights is None:
+        return out
+    T, K = handle.rank_row_map.shape
+    _require(recv_topk_weights.dtype == torch.float32 and recv_topk_weights.is_contiguous()
+             and recv_topk_weights.dim() == 2 and recv_topk_weights.shape[1] == K,
+             "recv_topk_weights must be contiguous float32 [rows, num_topk]")
+    out_w = torch.empty((T, K), dtype=torch.float32, device=y.device)
+    _lib.check(_lib.load().mi_ep_combine_rank_weights(
+        _ptr(recv_topk_weights), _ptr(handle.rank_row_map), T, K, recv_topk_weights.shape[0], _ptr(out_w),
+        _stream()), "mi_ep_combine_rank_weights")
+    return out, out_w
 
 
 def combine(y: torch.Tensor, slot_map: Union[torch.Tensor, DispatchHandle],

@@ -157,6 +157,49 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
                    float* recv_topk_weights, int* slot_map, int capacity_rows, void* stream);
 
 /*
+ * Dispatch de-duplicated by destination rank: the reference's own receive format (payload role
+ * of dispatch_impl, example080_deepep_jit_dispatch_payload/nv/empty_deepep_jit_dispatch_payload.cu:31-44,
+ * 241-256, then dispatch_copy_epilogue_impl without expansion,
+ * example081_deepep_jit_dispatch_copy_epilogue/nv/empty_deepep_jit_dispatch_copy_epilogue.cu:22-60).
+ * A token sends ONE row to every rank that owns at least one of its experts; rank r receives its
+ * rows in token order at [psum_rank_tokens[r-1], psum_rank_tokens[r]).
+ *   rank_slot_idx, rank_slot_base, num_tokens_per_rank   from mi_ep_dispatch_layout for the same topk_idx
+ *   expand_slot_map   NULL, or the slot_map of mi_ep_dispatch (rows of the expanded buffer)
+ *   recv_x / recv_scales   [capacity_rows, row_bytes] / float[capacity_rows, num_scales] or NULL
+ *   recv_topk_idx     int64[capacity_rows, num_topk] or NULL: the token's expert ids that live on
+ *                     the row's rank (minus rank * E/R when local_expert_ids != 0), -1 elsewhere
+ *   recv_topk_weights float[capacity_rows, num_topk] or NULL: the weights of those slots (1 when
+ *                     topk_weights is NULL), 0 elsewhere
+ *   recv_src_metadata int32[capacity_rows, 2 + num_topk] or NULL: {source_token_base + t, rank,
+ *                     then per slot the expanded row of the route when its expert lives on the
+ *                     rank and expand_slot_map is given, else -1} (column 0 as the reference's
+ *                     harness reads it, example080 build_and_run.py:733; source_token_base stands
+ *                     for rank_idx * num_max_tokens_per_rank)
+ *   rank_row_map      int32[num_tokens, num_topk]: the row that carries route (t,k); slots that
+ *                     share a rank share a row; -1 for non-routes and dropped rows
+ *   psum_rank_tokens  int32[num_ranks]: inclusive rows per rank
+ *                     (psum_num_recv_tokens_per_scaleup_rank, :734)
+ *   combine_map       int32[num_tokens, num_topk] or NULL: rank_row_map on the first slot of
+ *                     every distinct rank of the token, -1 elsewhere: each received row once.
+ *                     mi_ep_combine(y, rows, combine_map, topk_weights = NULL, ...) is then the
+ *                     reference's combine of this format (an ordered sum of the ranks' rows)
+ * Rows at or beyond capacity_rows are dropped; min(num_topk, num_ranks) * num_tokens always fit.
+ * mi_ep_combine_rank_weights returns the weights that travelled with the rows:
+ * [t,k] = recv_topk_weights[rank_row_map[t,k], k], 0 for non-routes (combined_topk_weights,
+ * example082 build_and_run.py:765).
+ */
+int mi_ep_dispatch_ranks(const void* x, const float* x_scales, const int64_t* topk_idx,
+                         const float* topk_weights, const int* rank_slot_idx, int rank_slot_base,
+                         const int* num_tokens_per_rank, const int* expand_slot_map, int num_tokens,
+                         int num_topk, int num_ranks, int num_experts, int row_bytes, int num_scales,
+                         int source_token_base, int local_expert_ids, void* recv_x, float* recv_scales,
+                         int64_t* recv_topk_idx, float* recv_topk_weights, int* recv_src_metadata,
+                         int* rank_row_map, int* combine_map, int* psum_rank_tokens, int capacity_rows,
+                         void* stream);
+int mi_ep_combine_rank_weights(const float* recv_topk_weights, const int* rank_row_map, int num_tokens,
+                               int num_topk, int num_rows, float* combined_topk_weights, void* stream);
+
+/*
  * Pull-mode dispatch with a map from an earlier dispatch (the reference's cached mode,
  * kCachedMode of dispatch_copy_epilogue_impl,
  * example081_deepep_jit_dispatch_copy_epilogue/nv/empty_deepep_jit_dispatch_copy_epilogue.cu:11,

@@ -26,6 +26,9 @@
  *   ep_oracle_permute           example081_deepep_jit_dispatch_copy_epilogue/nv/
  *                               empty_deepep_jit_dispatch_copy_epilogue.cu:22-60
  *                               (payload, scales, weights and source metadata per row)
+ *   ep_oracle_permute_ranks     example080 .cu:31-44,241-256 + example081 .cu:22-60 without expansion:
+ *                               one row per (token, destination rank), K ids / weights and the
+ *                               source metadata per row
  *   ep_oracle_gather_rows,
  *   ep_oracle_pull_indices      example056_thunderkitten_moe_dispatch_gemm_easy/nv/
  *                               empty_thunderkitten_moe_dispatch_gemm.cu:181-202,521-564
@@ -45,13 +48,17 @@
  *   channel prefix   closed form for the reference's routeDst pattern
  *   rank prefix      numpy cumsum over axis 0
  *   permute          numpy fancy-index gather
+ *   permute by rank  numpy: rows of rank r = x[flag[:, r]] in token order, masks from the ids;
+ *                    the reference harness's own checks (example080 build_and_run.py:728-748)
  *   pull indices     the closed form of the ThunderKittens example's own generator
  *   combine          exact rational arithmetic rounded once per fma (python ints),
  *                    integer-valued exact sums, K=1 copy, closed forms
  *   bf16 codec       exhaustive against torch.bfloat16 (fixtures in tests/golden)
  * Parity unpinned: the order in which two bias rows are added in the reference's
  * combine epilogue (its arithmetic lives in the un-vendored DeepEP tree); this
- * file defines it as acc + bias_0 + bias_1 after the top-k loop.
+ * file defines it as acc + bias_0 + bias_1 after the top-k loop.  Also unpinned, for the
+ * same reason: column 1 of recv_src_metadata (defined here as the destination rank) and
+ * whether recv_topk_idx holds global or rank-local expert ids (both offered).
  */
 #include <math.h>
 #include <stddef.h>
@@ -319,6 +326,91 @@ int ep_oracle_permute(const void* x, int row_bytes, const float* x_scales, int n
     size_t i = (size_t)t * num_topk + src_k[row];
     if (recv_topk_idx) recv_topk_idx[row] = topk_idx[i];
     if (recv_topk_weights) recv_topk_weights[row] = topk_weights[i];
+  }
+  return 0;
+}
+
+/*
+ * Dispatch de-duplicated by destination rank, the format of the reference's own dispatch
+ * (payload role of dispatch_impl, example080 .cu:31-44,241-256, followed by the copy epilogue
+ * without expansion, example081 .cu:22-60): a token sends ONE row to every rank that owns at
+ * least one of its experts.  Rank r receives its rows in token order at
+ * [psum[r-1], psum[r]) (psum inclusive, as psum_num_recv_tokens_per_scaleup_rank).  Per row n
+ * of token t on rank r:
+ *   recv_x / recv_scales   byte copy of the token's input
+ *   recv_topk_idx[n,k]     topk_idx[t,k] if that expert lives on r (minus r * E/R when
+ *                          local_expert_ids), else -1
+ *   recv_topk_weights[n,k] topk_weights[t,k] where recv_topk_idx[n,k] >= 0, else 0
+ *   recv_src_metadata[n,:] {source_token_base + t, r, then per slot k the row of route (t,k) in
+ *                          the expanded buffer (expand_slot_map, may be NULL) where the expert
+ *                          lives on r, else -1}
+ * and per token: rank_row_map[t,k] = the row that carries route (t,k) (-1 for non-routes;
+ * slots that share a rank share a row).  Rows at or beyond capacity_rows are dropped.
+ * Outputs other than recv_x and rank_row_map may be NULL.
+ */
+int ep_oracle_permute_ranks(const void* x, int row_bytes, const float* x_scales, int num_scales,
+                            const int64_t* topk_idx, const float* topk_weights, int num_tokens,
+                            int num_topk, int num_ranks, int num_experts, int source_token_base,
+                            int local_expert_ids, const int* expand_slot_map, int capacity_rows,
+                            void* recv_x, float* recv_scales, int64_t* recv_topk_idx,
+                            float* recv_topk_weights, int* recv_src_metadata, int* rank_row_map,
+                            int* psum_rank_tokens) {
+  if (num_ranks <= 0 || num_ranks > EP_MAX_RANKS || num_experts % num_ranks != 0) return -22;
+  const int per_rank = num_experts / num_ranks;
+  const int stride = 2 + num_topk;
+  const uint8_t* xin = (const uint8_t*)x;
+  uint8_t* xout = (uint8_t*)recv_x;
+  int count[EP_MAX_RANKS] = {0}, base[EP_MAX_RANKS + 1] = {0}, next[EP_MAX_RANKS] = {0};
+  for (int t = 0; t < num_tokens; ++t) {
+    int hit[EP_MAX_RANKS] = {0};
+    for (int k = 0; k < num_topk; ++k) {
+      int64_t e = topk_idx[(size_t)t * num_topk + k];
+      if (route_valid(e, num_experts)) hit[e / per_rank] = 1;
+    }
+    for (int r = 0; r < num_ranks; ++r) count[r] += hit[r];
+  }
+  for (int r = 0; r < num_ranks; ++r) {
+    base[r + 1] = base[r] + count[r];
+    if (psum_rank_tokens) psum_rank_tokens[r] = base[r + 1];
+  }
+  for (int t = 0; t < num_tokens; ++t) {
+    int row_of[EP_MAX_RANKS];
+    for (int r = 0; r < num_ranks; ++r) row_of[r] = -2;  /* not reached */
+    for (int k = 0; k < num_topk; ++k) {
+      size_t i = (size_t)t * num_topk + k;
+      int64_t e = topk_idx[i];
+      rank_row_map[i] = -1;
+      if (!route_valid(e, num_experts)) continue;
+      int r = (int)(e / per_rank);
+      if (row_of[r] == -2) {
+        int row = base[r] + next[r]++;
+        row_of[r] = row < capacity_rows ? row : -1;
+      }
+      rank_row_map[i] = row_of[r];
+    }
+    for (int r = 0; r < num_ranks; ++r) {
+      int row = row_of[r];
+      if (row < 0) continue;
+      memcpy(xout + (size_t)row * row_bytes, xin + (size_t)t * row_bytes, (size_t)row_bytes);
+      if (recv_scales)
+        memcpy(recv_scales + (size_t)row * num_scales, x_scales + (size_t)t * num_scales,
+               sizeof(float) * (size_t)num_scales);
+      if (recv_src_metadata) {
+        recv_src_metadata[(size_t)row * stride + 0] = source_token_base + t;
+        recv_src_metadata[(size_t)row * stride + 1] = r;
+      }
+      for (int k = 0; k < num_topk; ++k) {
+        size_t i = (size_t)t * num_topk + k;
+        int64_t e = topk_idx[i];
+        int local = route_valid(e, num_experts) && (int)(e / per_rank) == r;
+        if (recv_topk_idx)
+          recv_topk_idx[(size_t)row * num_topk + k] = local ? e - (local_expert_ids ? (int64_t)r * per_rank : 0) : -1;
+        if (recv_topk_weights)
+          recv_topk_weights[(size_t)row * num_topk + k] = local ? (topk_weights ? topk_weights[i] : 1.0f) : 0.0f;
+        if (recv_src_metadata)
+          recv_src_metadata[(size_t)row * stride + 2 + k] = (local && expand_slot_map) ? expand_slot_map[i] : -1;
+      }
+    }
   }
   return 0;
 }

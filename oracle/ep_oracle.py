@@ -166,6 +166,40 @@ def permute(x_bytes: np.ndarray, scales, topk_idx, topk_weights, src_map, src_k,
     return recv_x, recv_scales, recv_idx, recv_w
 
 
+def permute_ranks(x_bytes: np.ndarray, scales, topk_idx, topk_weights, num_ranks: int, num_experts: int,
+                  source_token_base: int = 0, local_expert_ids: bool = False, expand_slot_map=None,
+                  capacity_rows=None):
+    """Dispatch de-duplicated by destination rank; returns a dict (arrays trimmed to the row total)."""
+    topk_idx = _c(topk_idx, np.int64)
+    T, K = topk_idx.shape
+    x_bytes = _c(x_bytes, np.uint8)
+    row_bytes = x_bytes.shape[1]
+    scales = None if scales is None else _c(scales, np.float32)
+    S = 0 if scales is None else scales.shape[1]
+    topk_weights = None if topk_weights is None else _c(topk_weights, np.float32)
+    expand_slot_map = None if expand_slot_map is None else _c(expand_slot_map, np.int32)
+    cap = T * min(K, num_ranks) if capacity_rows is None else capacity_rows
+    out = dict(recv_x=np.zeros((cap, row_bytes), dtype=np.uint8),
+               recv_scales=None if scales is None else np.zeros((cap, S), dtype=np.float32),
+               recv_topk_idx=np.full((cap, K), -9, dtype=np.int64),
+               recv_topk_weights=np.full((cap, K), -9.0, dtype=np.float32),
+               recv_src_metadata=np.full((cap, 2 + K), -9, dtype=np.int32),
+               rank_row_map=np.empty((T, K), dtype=np.int32),
+               psum_rank_tokens=np.empty(num_ranks, dtype=np.int32))
+    rc = _load().ep_oracle_permute_ranks(
+        _p(x_bytes), row_bytes, _p(scales), S, _p(topk_idx), _p(topk_weights), T, K, num_ranks, num_experts,
+        source_token_base, 1 if local_expert_ids else 0, _p(expand_slot_map), cap, _p(out["recv_x"]),
+        _p(out["recv_scales"]), _p(out["recv_topk_idx"]), _p(out["recv_topk_weights"]),
+        _p(out["recv_src_metadata"]), _p(out["rank_row_map"]), _p(out["psum_rank_tokens"]))
+    if rc != 0:
+        raise ValueError(f"ep_oracle_permute_ranks: {rc}")
+    rows = min(int(out["psum_rank_tokens"][-1]), cap)
+    for key in ("recv_x", "recv_scales", "recv_topk_idx", "recv_topk_weights", "recv_src_metadata"):
+        if out[key] is not None:
+            out[key] = out[key][:rows]
+    return out
+
+
 def gather_rows(x_bytes: np.ndarray, scales, src_map: np.ndarray):
     x_bytes = _c(x_bytes, np.uint8)
     src_map = _c(src_map, np.int32)
