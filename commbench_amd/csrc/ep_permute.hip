@@ -27,8 +27,9 @@ constexpr int kPushWaves = kPushThreads / kWave;
 // for the routing tables.
 constexpr int kDies = 8;
 constexpr size_t kTileSourceBytesMax = 3840u * 1024u;
-constexpr size_t kRunBytesMin = 96u * 1024u;  // expected bytes a tile sends to one expert
-constexpr size_t kRowBytesMin = 12u * 1024u;
+constexpr size_t kRowBytesMin = 4u * 1024u;
+constexpr size_t kFatRowBytesMax = 12u * 1024u;  // below this, 8 KiB instead of 2 KiB per workgroup
+constexpr int kRunRowsMin = 4;
 // The first workgroups of a tile pull its source rows into L2, 8 rows per group of workgroups.
 constexpr int kPrefetchGroups = 32;
 
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
 // Launched as a 3-D grid (x = part of the row * 8 + die, y = entry of the tile's list, z = round
 // of eight tiles) so that no index needs a division: a wave moves only 1 KiB, which leaves it
 // a budget of about a hundred vector instructions before instruction issue, not HBM, sets the pace.
-template <bool kStreamStores>
+template <bool kStreamStores, int kVecs>
 __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const PermuteArgs a, const int num_tiles,
                                                                        const int prefetch_ys) {
   const int lane = lane_id();
@@ -131,15 +132,19 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
     // when the rows come from HBM (not from the memory-side cache) this keeps their reads from
     // being sprinkled over the whole tile, where they would break up the runs of writes
     // (measured at 8192 x 14 KiB rows: 182 us against 208 us; 2-3 us lost when the rows are cached).
-    const int v = (part * kPushWaves + wave) * kWave + lane;
+    const int v0 = (part * kPushWaves + wave) * (kWave * kVecs) + lane;
     const int rows_per_y = kTileTokens / prefetch_ys;
     const int row0 = tile * kTileTokens + static_cast<int>(blockIdx.y) * rows_per_y;
     uint32_t fold = 0;
-    if (v < a.row_vecs) {
-      for (int i = 0; i < rows_per_y; ++i) {
-        if (row0 + i < a.num_tokens) {
-          const vec16 q = a.x[static_cast<size_t>(row0 + i) * a.row_vecs + v];
-          fold ^= q[0] ^ q[1] ^ q[2] ^ q[3];
+    for (int i = 0; i < rows_per_y; ++i) {
+      if (row0 + i < a.num_tokens) {
+#pragma unroll
+        for (int u = 0; u < kVecs; ++u) {
+          const int v = v0 + u * kWave;
+          if (v < a.row_vecs) {
+            const vec16 q = a.x[static_cast<size_t>(row0 + i) * a.row_vecs + v];
+            fold ^= q[0] ^ q[1] ^ q[2] ^ q[3];
+          }
         }
       }
     }
@@ -161,9 +166,13 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
   if (flat < first_flat || flat >= first_flat + routes || token < 0 || token >= a.num_tokens) return;
   const bool routed = expert >= 0 && expert < a.num_experts && rel >= 0;
 
-  const int v = (part * kPushWaves + wave) * kWave + lane;
-  vec16 buf = {0u, 0u, 0u, 0u};
-  if (routed && v < a.row_vecs) buf = a.x[static_cast<size_t>(token) * a.row_vecs + v];
+  const int v0 = (part * kPushWaves + wave) * (kWave * kVecs) + lane;
+  vec16 buf[kVecs];
+#pragma unroll
+  for (int u = 0; u < kVecs; ++u) {
+    const int v = v0 + u * kWave;
+    if (routed && v < a.row_vecs) buf[u] = a.x[static_cast<size_t>(token) * a.row_vecs + v];
+  }
 
   int slot = -1;
   if (routed) {
@@ -185,12 +194,18 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
         a.recv_scales[static_cast<size_t>(slot) * a.num_scales + j] =
             a.x_scales[static_cast<size_t>(token) * a.num_scales + j];
   }
-  if (slot >= 0 && v < a.row_vecs) {
-    vec16* dst = a.recv_x + static_cast<size_t>(slot) * a.row_vecs + v;
-    if (kStreamStores)
-      __builtin_nontemporal_store(buf, dst);
-    else
-      *dst = buf;
+  if (slot >= 0) {
+#pragma unroll
+    for (int u = 0; u < kVecs; ++u) {
+      const int v = v0 + u * kWave;
+      if (v < a.row_vecs) {
+        vec16* dst = a.recv_x + static_cast<size_t>(slot) * a.row_vecs + v;
+        if (kStreamStores)
+          __builtin_nontemporal_store(buf[u], dst);
+        else
+          *dst = buf[u];
+      }
+    }
   }
 }
 
@@ -458,18 +473,17 @@ __global__ __launch_bounds__(256) void ep_write_yardstick_kernel(vec16* __restri
 }  // namespace
 
 // Destination order pays when every die has work in (nearly) every round, a tile's rows fit L2,
-// and a tile leaves an expert a run of adjacent rows long enough for the memory controllers to
-// notice.  Measured: 14 KiB rows in 112 KiB runs gain 13-16 %, 8 KiB rows in 128 KiB runs gain
-// nothing, 7 KiB rows in 56 KiB runs lose 8 %.
+// rows are long enough for a workgroup to have something to move and a tile leaves an expert a
+// run of several adjacent rows.  Measured against the token-major kernel, whole copy:
+// 14 KiB rows -13..-16 %, 8 KiB rows -8..-13 %, 4 KiB rows -13 %, 6-7 KiB rows -3..0 %.
 bool destination_order_pays(const PermuteArgs& a) {
   const int tiles = (a.num_tokens + kTileTokens - 1) / kTileTokens;
   const int rounds = (tiles + kDies - 1) / kDies;
   if (tiles * 8 < rounds * kDies * 7) return false;  // more than 1/8 of the die-rounds idle
   const size_t row_bytes = static_cast<size_t>(a.row_vecs) * sizeof(vec16);
   if (kTileTokens * row_bytes > kTileSourceBytesMax) return false;
-  if (row_bytes < kRowBytesMin) return false;  // 7 and 8 KiB rows measured no gain
-  const size_t run_bytes = static_cast<size_t>(kTileTokens) * a.num_topk * row_bytes / a.num_experts;
-  return run_bytes >= kRunBytesMin;
+  if (row_bytes < kRowBytesMin) return false;
+  return kTileTokens * a.num_topk >= kRunRowsMin * a.num_experts;  // expected rows per (tile, expert)
 }
 
 hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream) {
@@ -480,15 +494,22 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
   if (by_destination) {
     const int tiles = (a.num_tokens + kTileTokens - 1) / kTileTokens;
     const int rounds = (tiles + kDies - 1) / kDies;
-    const int per_workgroup = kPushWaves * kWave;
+    // Long rows: 2 KiB per workgroup, seven workgroups on a 14 KiB row.  Short rows do better with
+    // 8 KiB per workgroup (one or two per row): fewer, fatter workgroups for the same bytes.
+    const bool fat = static_cast<size_t>(a.row_vecs) * sizeof(vec16) < kFatRowBytesMax;
+    const int per_workgroup = kPushWaves * kWave * (fat ? 4 : 1);
     const int parts = (a.row_vecs + per_workgroup - 1) / per_workgroup;
     if (rounds > 65535 || parts * kDies > 65535) return hipErrorInvalidValue;
     const int prefetch_ys = kPrefetchGroups;
-    hipLaunchKernelGGL((ep_permute_tiles_kernel<true>),
-                       dim3(static_cast<unsigned>(parts * kDies),
-                            static_cast<unsigned>(kTileTokens * a.num_topk + prefetch_ys),
-                            static_cast<unsigned>(rounds)),
-                       dim3(kPushThreads), 0, stream, a, tiles, prefetch_ys);
+    const dim3 grid(static_cast<unsigned>(parts * kDies),
+                    static_cast<unsigned>(kTileTokens * a.num_topk + prefetch_ys),
+                    static_cast<unsigned>(rounds));
+    if (fat)
+      hipLaunchKernelGGL((ep_permute_tiles_kernel<true, 4>), grid, dim3(kPushThreads), 0, stream, a, tiles,
+                         prefetch_ys);
+    else
+      hipLaunchKernelGGL((ep_permute_tiles_kernel<true, 1>), grid, dim3(kPushThreads), 0, stream, a, tiles,
+                         prefetch_ys);
     return hipGetLastError();
   }
   const int batches = (a.row_vecs + kWave - 1) / kWave;

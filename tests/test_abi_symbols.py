@@ -50,9 +50,10 @@ def test_host_only_entry_points():
     # destination order: long rows, enough tiles for all eight dies, long enough runs per expert
     assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 14336) == 2
     assert lib.mi_ep_dispatch_schedule_for(4096, 8, 256, 14336) == 2
-    assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 7168) == 1      # 7 KiB rows
+    assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 7168) == 2
+    assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 2048) == 1      # 2 KiB rows
     assert lib.mi_ep_dispatch_schedule_for(1024, 8, 256, 14336) == 1     # 4 tiles for 8 dies
-    assert lib.mi_ep_dispatch_schedule_for(8192, 2, 1024, 14336) == 1    # runs of 7 KiB per expert
+    assert lib.mi_ep_dispatch_schedule_for(8192, 2, 1024, 14336) == 1    # half a row per tile and expert
     assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 16384) == 1     # a tile's rows exceed L2
     assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 100) == -22
     assert lib.mi_ep_workspace_bytes(8192, 8, 256, 9) == 0       # more than 8 ranks

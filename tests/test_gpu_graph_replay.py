@@ -13,8 +13,18 @@ from . import gpu_util as gu
 pytestmark = pytest.mark.gpu
 
 
-def test_graph_replays_match_eager(oracle):
+@pytest.fixture(params=[gu.SCHEDULE_BY_TOKEN, gu.SCHEDULE_BY_DESTINATION], ids=["by_token", "by_destination"])
+def schedule(request):
+    """Forces one of the two copy kernels for the duration of a test (captured graphs keep it)."""
+    lib = _lib.load()
+    assert lib.mi_ep_set_dispatch_schedule(request.param) == 0
+    yield request.param
+    assert lib.mi_ep_set_dispatch_schedule(gu.SCHEDULE_AUTO) == 0
+
+
+def test_graph_replays_match_eager(oracle, schedule):
     T, K, E, R, H = 3000, 8, 64, 8, 1024
+    print(f"schedule {schedule}", flush=True)
     rng = np.random.default_rng(12)
     lib = _lib.load()
     dev = gu.DEV
