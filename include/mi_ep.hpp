@@ -93,11 +93,16 @@ struct DispatchHandle {
   int* psum_rank_rows = nullptr;         // [R]
   int* channel_prefix_matrix = nullptr;  // [R, C] (C = num_channels of the buffer, may be 0)
   int* slot_rel = nullptr;               // [T, K]
+  int* rank_slot_idx = nullptr;          // [T, K] the deterministic prologue's table (base 0)
   int* route_order = nullptr;            // [tiles * 256 * K, 4] routes in destination order
   int* slot_map = nullptr;               // [T, K]
   int* recv_src_map = nullptr;           // [capacity]
   int64_t* recv_topk_idx = nullptr;      // [capacity]
   float* recv_topk_weights = nullptr;    // [capacity]
+  // per-rank receive format (dispatch_ranks)
+  int* rank_row_map = nullptr;           // [T, K] row carrying each route
+  int* rank_combine_map = nullptr;       // [T, K] each received row once
+  int* psum_rank_tokens = nullptr;       // [R] inclusive rows per rank
 };
 
 // Owns the layout workspace and the handle's index arrays; payload buffers stay with the caller.
@@ -126,6 +131,10 @@ class ExpertParallelBuffer {
     if (num_channels > 0)
       MI_EP_HIP_CHECK(hipMalloc(&h_.channel_prefix_matrix, sizeof(int) * num_ranks * num_channels));
     MI_EP_HIP_CHECK(hipMalloc(&h_.slot_rel, sizeof(int) * (tk + 1)));
+    MI_EP_HIP_CHECK(hipMalloc(&h_.rank_slot_idx, sizeof(int) * (tk + 1)));
+    MI_EP_HIP_CHECK(hipMalloc(&h_.rank_row_map, sizeof(int) * (tk + 1)));
+    MI_EP_HIP_CHECK(hipMalloc(&h_.rank_combine_map, sizeof(int) * (tk + 1)));
+    MI_EP_HIP_CHECK(hipMalloc(&h_.psum_rank_tokens, sizeof(int) * num_ranks));
     MI_EP_HIP_CHECK(hipMalloc(&h_.route_order, mi_ep_route_order_bytes(num_max_tokens, num_topk) + 16));
     MI_EP_HIP_CHECK(hipMalloc(&h_.slot_map, sizeof(int) * (tk + 1)));
     MI_EP_HIP_CHECK(hipMalloc(&h_.recv_src_map, sizeof(int) * (capacity_ + 1)));
@@ -138,6 +147,7 @@ class ExpertParallelBuffer {
   ~ExpertParallelBuffer() {
     void* owned[] = {workspace_, h_.num_tokens_per_rank, h_.num_tokens_per_expert, h_.is_token_in_rank,
                      h_.expert_offsets, h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel,
+                     h_.rank_slot_idx, h_.rank_row_map, h_.rank_combine_map, h_.psum_rank_tokens,
                      h_.route_order, h_.slot_map, h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights};
     for (void* p : owned)
       if (p != nullptr) (void)hipFree(p);
@@ -150,14 +160,16 @@ class ExpertParallelBuffer {
   const DispatchHandle& handle() const { return h_; }
 
   // Fused layout: counts, flags, offsets, per-route segment positions (and channel prefixes).
-  const DispatchHandle& get_dispatch_layout(const TopkIdx* d_topk_idx, int num_tokens, hipStream_t stream = 0) {
+  // with_rank_slots also fills rank_slot_idx, the deterministic prologue's per-rank slot table.
+  const DispatchHandle& get_dispatch_layout(const TopkIdx* d_topk_idx, int num_tokens, hipStream_t stream = 0,
+                                            bool with_rank_slots = false) {
     check_tokens(num_tokens);
     h_.num_tokens = num_tokens;
     MI_EP_CHECK(mi_ep_dispatch_layout(d_topk_idx, num_tokens, num_topk_, num_ranks_, num_experts_,
                                       h_.expert_alignment, num_channels_, h_.num_tokens_per_rank,
                                       h_.num_tokens_per_expert, h_.is_token_in_rank, h_.expert_offsets,
                                       h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel,
-                                      /*rank_slot_idx=*/nullptr, /*rank_slot_base=*/0, h_.route_order,
+                                      with_rank_slots ? h_.rank_slot_idx : nullptr, /*rank_slot_base=*/0, h_.route_order,
                                       workspace_, workspace_bytes_, stream));
     return h_;
   }
@@ -173,6 +185,33 @@ class ExpertParallelBuffer {
                                h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights, h_.slot_map,
                                capacity_, stream));
     return h_;
+  }
+
+  // The reference's own receive format: one row per (token, destination rank), ranks' rows in token
+  // order.  Outputs hold rank_capacity_rows() rows; any of the three side arrays may be null.
+  // source_token_base stands for rank_idx * num_max_tokens_per_rank in the metadata's column 0.
+  const DispatchHandle& dispatch_ranks(const void* d_x, const float* d_scales, const TopkIdx* d_topk_idx,
+                                       const float* d_topk_weights, int num_tokens, int row_bytes,
+                                       int num_scales, int source_token_base, bool local_expert_ids,
+                                       void* d_recv_x, float* d_recv_scales, int64_t* d_recv_topk_idx,
+                                       float* d_recv_topk_weights, int* d_recv_src_metadata,
+                                       hipStream_t stream = 0) {
+    get_dispatch_layout(d_topk_idx, num_tokens, stream, /*with_rank_slots=*/true);
+    MI_EP_CHECK(mi_ep_dispatch_ranks(d_x, d_scales, d_topk_idx, d_topk_weights, h_.rank_slot_idx, 0,
+                                     h_.num_tokens_per_rank, nullptr, num_tokens, num_topk_, num_ranks_,
+                                     num_experts_, row_bytes, num_scales, source_token_base,
+                                     local_expert_ids ? 1 : 0, d_recv_x, d_recv_scales, d_recv_topk_idx,
+                                     d_recv_topk_weights, d_recv_src_metadata, h_.rank_row_map,
+                                     h_.rank_combine_map, h_.psum_rank_tokens, rank_capacity_rows(), stream));
+    return h_;
+  }
+  int rank_capacity_rows() const { return max_tokens_ * (num_topk_ < num_ranks_ ? num_topk_ : num_ranks_); }
+
+  // The reference's combine of that format: the ordered sum of the rows a token sent out (+ biases).
+  void combine_ranks(const void* d_y, int num_rows, const void* d_bias_0, const void* d_bias_1, int hidden,
+                     void* d_combined_x, hipStream_t stream = 0) const {
+    MI_EP_CHECK(mi_ep_combine(d_y, num_rows, h_.rank_combine_map, nullptr, d_bias_0, d_bias_1, nullptr,
+                              h_.num_tokens, num_topk_, hidden, d_combined_x, nullptr, stream));
   }
 
   // combined_x[t] = bf16(sum_k w[t,k] * y[slot_map[t,k]] + bias_0 + bias_1); null weights = plain sum.

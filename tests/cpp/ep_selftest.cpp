@@ -25,6 +25,8 @@ int ep_oracle_slot_maps(const int64_t*, int, int, int, const int*, int*, int*, i
 int ep_oracle_channel_prefix(const uint8_t*, int, int, int, int*);
 int ep_oracle_permute(const void*, int, const float*, int, const int64_t*, const float*, int, const int*,
                       const int*, int, void*, float*, int64_t*, float*, int);
+int ep_oracle_permute_ranks(const void*, int, const float*, int, const int64_t*, const float*, int, int, int, int, int,
+                            int, const int*, int, void*, float*, int64_t*, float*, int*, int*, int*);
 int ep_oracle_combine(const uint16_t*, const int*, const float*, const uint16_t*, const uint16_t*, int, int,
                       int, uint16_t*, int);
 uint16_t ep_oracle_f32_to_bf16(float);
@@ -208,6 +210,61 @@ bool check_round_trip() {
   return ok;
 }
 
+// The reference's own receive format (one row per token and destination rank) and its combine.
+bool check_rank_format() {
+  Case c{517, 8, 8, 64, kRankSweep};
+  const int hidden = 264, row_bytes = hidden * 2, stride = 2 + c.topk, base = 3 * 1024;
+  std::vector<TopkIdx> idx = make_topk(c);
+  for (size_t i = 0; i < idx.size(); i += 11) idx[i] = -1;
+  std::vector<float> w(idx.size());
+  for (size_t i = 0; i < w.size(); ++i) w[i] = 0.0625f * static_cast<float>(1 + (i * 5) % 13);
+  std::vector<uint16_t> x(static_cast<size_t>(c.tokens) * hidden);
+  for (size_t i = 0; i < x.size(); ++i) x[i] = ep_oracle_f32_to_bf16(static_cast<float>(static_cast<int>((i * 2246822519u) >> 21 & 511) - 256) / 32.0f);
+  mi_ep::ExpertParallelBuffer buf(c.tokens, c.topk, c.experts, c.ranks);
+  const int cap = buf.rank_capacity_rows();
+  std::vector<uint16_t> want_recv(static_cast<size_t>(cap) * hidden), want_out(x.size());
+  std::vector<int64_t> want_idx(static_cast<size_t>(cap) * c.topk);
+  std::vector<float> want_w(static_cast<size_t>(cap) * c.topk);
+  std::vector<int> want_meta(static_cast<size_t>(cap) * stride), want_map(idx.size()), want_psum(c.ranks);
+  ep_oracle_permute_ranks(x.data(), row_bytes, nullptr, 0, idx.data(), w.data(), c.tokens, c.topk, c.ranks, c.experts,
+                          base, 1, nullptr, cap, want_recv.data(), nullptr, want_idx.data(), want_w.data(),
+                          want_meta.data(), want_map.data(), want_psum.data());
+  const int rows = want_psum.back();
+
+  DeviceArray<TopkIdx> d_idx(idx.size());
+  DeviceArray<float> d_w(w.size()), d_recv_w(want_w.size());
+  DeviceArray<uint16_t> d_x(x.size()), d_out(x.size()), d_recv(want_recv.size());
+  DeviceArray<int64_t> d_recv_idx(want_idx.size());
+  DeviceArray<int> d_meta(want_meta.size());
+  d_idx.upload(idx);
+  d_w.upload(w);
+  d_x.upload(x);
+  const mi_ep::DispatchHandle& h = buf.dispatch_ranks(d_x.p, nullptr, d_idx.p, d_w.p, c.tokens, row_bytes, 0, base, true,
+                                                      d_recv.p, nullptr, d_recv_idx.p, d_recv_w.p, d_meta.p);
+  buf.combine_ranks(d_recv.p, cap, nullptr, nullptr, hidden, d_out.p);
+  buf.check_status();
+  auto head = [](auto v, size_t n) { v.resize(n); return v; };
+  bool ok = head(d_recv.download(want_recv.size()), static_cast<size_t>(rows) * hidden) == head(want_recv, static_cast<size_t>(rows) * hidden);
+  ok = ok && head(d_recv_idx.download(want_idx.size()), static_cast<size_t>(rows) * c.topk) == head(want_idx, static_cast<size_t>(rows) * c.topk);
+  ok = ok && head(d_recv_w.download(want_w.size()), static_cast<size_t>(rows) * c.topk) == head(want_w, static_cast<size_t>(rows) * c.topk);
+  ok = ok && head(d_meta.download(want_meta.size()), static_cast<size_t>(rows) * stride) == head(want_meta, static_cast<size_t>(rows) * stride);
+  std::vector<int> got_map(want_map.size()), got_combine(want_map.size()), got_psum(c.ranks);
+  MI_EP_HIP_CHECK(hipMemcpy(got_map.data(), h.rank_row_map, got_map.size() * sizeof(int), hipMemcpyDeviceToHost));
+  MI_EP_HIP_CHECK(hipMemcpy(got_combine.data(), h.rank_combine_map, got_combine.size() * sizeof(int), hipMemcpyDeviceToHost));
+  MI_EP_HIP_CHECK(hipMemcpy(got_psum.data(), h.psum_rank_tokens, got_psum.size() * sizeof(int), hipMemcpyDeviceToHost));
+  ok = ok && got_map == want_map && got_psum == want_psum;
+  // the ordered sum over the rows the checker says each token sent out
+  ep_oracle_combine(want_recv.data(), got_combine.data(), nullptr, nullptr, nullptr, c.tokens, c.topk, hidden,
+                    want_out.data(), 1);
+  ok = ok && d_out.download(want_out.size()) == want_out;
+  // each received row exactly once in the combine map
+  std::vector<int> seen(rows, 0);
+  for (int r : got_combine)
+    if (r >= 0 && r < rows) ++seen[r];
+  for (int n : seen) ok = ok && n == 1;
+  return ok;
+}
+
 struct MetricRow {
   std::string surface;
   Case c;
@@ -337,6 +394,11 @@ int main(int argc, char** argv) {
   {
     const bool ok = check_round_trip();
     if (!ok) std::cerr << "FAIL dispatch/combine round trip\n";
+    pass = pass && ok;
+  }
+  {
+    const bool ok = check_rank_format();
+    if (!ok) std::cerr << "FAIL per-rank dispatch format\n";
     pass = pass && ok;
   }
 
