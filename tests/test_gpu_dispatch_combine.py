@@ -136,6 +136,26 @@ def test_permute_ragged_shapes(oracle, shape):
     dispatch_and_check(oracle, (E, R), topk_np, w_np, x_cpu, scales_cpu, align=1)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_permute_random_shapes(oracle, seed):
+    """Shapes drawn at random (tile remainders, tile counts that do not divide by eight, masked and
+    out-of-range ids, duplicates, alignment pads, scales), both copy kernels, bit-exact."""
+    rng = np.random.default_rng(1000 + seed)
+    T = int(rng.integers(1, 6000))
+    K = int(rng.integers(1, 9))
+    R = int(rng.choice([1, 2, 4, 8]))
+    E = R * int(rng.integers(1, 1024 // R + 1 if seed % 3 == 0 else 17))
+    row_bytes = 16 * int(rng.integers(1, 80))
+    S = int(rng.integers(0, 9))
+    align = int(rng.choice([1, 1, 3, 16, 128]))
+    print(f"seed {seed}: T={T} K={K} R={R} E={E} row_bytes={row_bytes} S={S} align={align}", flush=True)
+    topk_np = rng.integers(-2, E + 2, size=(T, K)).astype(np.int64)
+    w_np = rng.standard_normal((T, K)).astype(np.float32)
+    x_cpu = torch.from_numpy(rng.integers(0, 256, size=(T, row_bytes), dtype=np.uint8))
+    scales_cpu = torch.from_numpy(rng.standard_normal((T, S)).astype(np.float32)) if S else None
+    dispatch_and_check(oracle, (E, R), topk_np, w_np, x_cpu, scales_cpu, align=align)
+
+
 def test_capacity_limits_writes(oracle):
     """Rows at or beyond capacity_rows are dropped: never written, slot_map = -1."""
     rng = np.random.default_rng(3)
