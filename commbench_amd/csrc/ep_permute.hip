@@ -112,7 +112,8 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
 // consecutive rows of recv_x: a tile leaves ~256*K/E adjacent rows per expert, which the
 // memory controllers take far better than rows scattered one by one.  Sources are then
 // read once per route, K times per token; that only pays because tile j goes to
-// accelerator die j % 8 (workgroup b is dispatched to die b % 8) and a tile's 256 rows
+// accelerator die j % 8 (workgroup b is dispatched to die b % 8: read back from the XCC_ID
+// register, every workgroup of a 3-D grid sat on die (linear id) % 8) and a tile's 256 rows
 // fit that die's 4 MiB L2, so the repeats never leave the die.  A workgroup copies
 // kPushWaves KiB of one route's row; part 0 also writes the row's side data.
 // Launched as a 3-D grid (x = part of the row * 8 + die, y = entry of the tile's list, z = round
