@@ -400,7 +400,21 @@ def main():
                 owk.step()
             torch.cuda.synchronize()
             us = (time.perf_counter() - t0) * 1e6 / 100
+            omarks = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(30)]
+            for ev in omarks:
+                ev[0].record()
+                owk.layout()
+                ev[1].record()
+                owk.dispatch()
+                ev[2].record()
+                owk.combine()
+                ev[3].record()
+            torch.cuda.synchronize()
+            median = lambda i: sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for ev in omarks)[len(omarks) // 2]
             others[name] = {"us_per_step": us, "tokens_per_s": ocfg.num_tokens / (us * 1e-6),
+                            "kernel_us_median": {"layout": median(0), "dispatch": median(1), "combine": median(2)},
+                            "dispatch_schedule": owk.lib.mi_ep_dispatch_schedule_for(
+                                ocfg.num_tokens, ocfg.num_topk, ocfg.num_experts, ocfg.row_bytes),
                             "hbm_gbps_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9,
                             "hbm_frac_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS,
                             "num_routes": owk.num_routes}
