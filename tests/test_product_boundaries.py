@@ -37,3 +37,21 @@ def test_hip_sources_are_gfx950_only():
         text = open(path).read()
         assert "__HIP_PLATFORM_AMD__" not in text and "__CUDACC__" not in text, path
         assert "cuda_runtime" not in text and "triton" not in text.lower(), path
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU; asking for more exits with a message, before any GPU work."""
+    import subprocess
+    import sys
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                          capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 2
+    assert "one GPU only" in proc.stderr and proc.stdout.strip() == ""
+
+
+def test_host_twins_stay_out_of_the_device_entry_points():
+    """Only ep_host.hip may allocate or copy; the device entry points enqueue and return."""
+    for name in ("ep_abi.hip", "ep_layout.hip", "ep_permute.hip", "ep_combine.hip"):
+        text = open(os.path.join(PKG, "csrc", name)).read()
+        text = re.sub(r"//.*", "", text)
+        assert "hipMalloc" not in text and "hipFree" not in text and "hipMemset" not in text, name
