@@ -117,3 +117,22 @@ def test_dispatch_ranks_zero_tokens(oracle):
     x = torch.zeros((0, 64), dtype=torch.bfloat16, device=gu.DEV)
     _, _, _, h = ops.dispatch_ranks(buf, x, None, topk, None)
     assert h.psum_rank_tokens.cpu().tolist() == [0, 0]
+
+
+def test_dispatch_ranks_at_a_benchmark_shape(oracle):
+    """4096 tokens x 7168 bf16, 256 experts, top-8, 8 ranks (the c2 shape): about 5.25 rows per
+    token, compared whole with the checker, then combined back."""
+    cfg = wl.CONFIGS["c2"]
+    topk_np, w_np = wl.make_routing(cfg)
+    rng = np.random.default_rng(2)
+    x_cpu = wl.bf16_normal(rng, cfg.num_tokens, cfg.hidden)
+    recv_x, _, recv_w, h, ref = run_and_check(oracle, topk_np, w_np, x_cpu, None, cfg.num_experts, cfg.num_ranks,
+                                              local_ids=True, expand=True)
+    rows = h.num_recv_rows()
+    assert 5.0 * cfg.num_tokens < rows < 5.5 * cfg.num_tokens
+    out, out_w = ops.combine_ranks(recv_x, h, recv_w)
+    torch.cuda.synchronize()
+    first = oracle.rank_slots(topk_np, cfg.num_ranks, cfg.num_experts, 0) >= 0
+    want = oracle.combine(ref["recv_x"].view(np.uint16), np.where(first, ref["rank_row_map"], -1), num_threads=8)
+    assert gu.bf16_ulp_distance(gu.bf16_bits(out), want).max() <= 2
+    np.testing.assert_array_equal(out_w.cpu().numpy(), w_np)
