@@ -25,7 +25,7 @@ SIGNATURES = {
                                      _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _size, _vp]),
     "mi_ep_route_order_bytes": (_size, [_int, _int]),
     "mi_ep_dispatch": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int,
-                              _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
+                              _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
     "mi_ep_dispatch_ranks": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _int, _int, _int, _int, _int,
                                     _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
     "mi_ep_combine_rank_weights": (_int, [_vp, _vp, _int, _int, _int, _vp, _vp]),

@@ -195,7 +195,8 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
                    const int* route_order, const int* num_tokens_per_expert, int num_tokens, int num_topk,
                    int num_experts, int expert_alignment, int row_bytes, int num_scales,
                    void* recv_x, float* recv_scales, int* recv_src_map, int64_t* recv_topk_idx,
-                   float* recv_topk_weights, int* slot_map, int capacity_rows, void* stream) {
+                   float* recv_topk_weights, int* slot_map, int capacity_rows, int flags,
+                   void* stream) {
   if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK) return MI_EP_EINVAL;
   if (num_experts <= 0 || num_experts > MI_EP_MAX_EXPERTS || expert_alignment < 1) return MI_EP_EINVAL;
   if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
@@ -208,6 +209,7 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
   if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
   if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
   if (expert_alignment > 1 && num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
+  if ((flags & ~MI_EP_DISPATCH_KEEP_PAD_PAYLOAD) != 0) return MI_EP_EINVAL;
 
   PermuteArgs a{};
   a.x = static_cast<const vec16*>(x);
@@ -232,7 +234,7 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
   a.capacity_rows = capacity_rows;
   hipStream_t s = as_stream(stream);
   hipError_t e = launch_permute(a, g_permute_schedule.load(std::memory_order_relaxed), s);
-  if (e == hipSuccess && expert_alignment > 1) e = launch_pad_rows(a, s);
+  if (e == hipSuccess && expert_alignment > 1) e = launch_pad_rows(a, expert_alignment, (flags & MI_EP_DISPATCH_KEEP_PAD_PAYLOAD) == 0, s);
   return status_of(e);
 }
 

@@ -102,7 +102,7 @@ hipError_t launch_gather_rows(const vec16* x, const float* x_scales, const int* 
                               hipStream_t stream);
 hipError_t launch_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_source_rank,
                                int* pull_indices, hipStream_t stream);
-hipError_t launch_pad_rows(const PermuteArgs& a, hipStream_t stream);
+hipError_t launch_pad_rows(const PermuteArgs& a, int expert_alignment, bool zero_payload, hipStream_t stream);
 
 // Dispatch de-duplicated by destination rank: one row per (token, rank that owns one of its experts).
 struct RankPermuteArgs {

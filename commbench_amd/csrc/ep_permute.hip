@@ -320,20 +320,24 @@ __global__ __launch_bounds__(256) void ep_gather_rank_weights_kernel(const float
 }
 
 // Zero-fills the rows that expert_alignment > 1 leaves between a segment's last
-// route and the next segment.  One workgroup per expert.
-__global__ __launch_bounds__(kPermuteThreads) void ep_pad_rows_kernel(const PermuteArgs a) {
+// route and the next segment.  Workgroup (e, j) takes pad rows j, j + gridDim.y, ... of
+// expert e: at alignment 128 the pads are a fifth of the buffer, so they are spread over
+// the whole device rather than walked by one workgroup per expert.
+__global__ __launch_bounds__(kPermuteThreads) void ep_pad_rows_kernel(const PermuteArgs a, const bool zero_payload) {
   const int e = static_cast<int>(blockIdx.x);
   const int begin = a.expert_offsets[e] + a.num_tokens_per_expert[e];
   int end = a.expert_offsets[e + 1];
   if (end > a.capacity_rows) end = a.capacity_rows;
   const int tid = static_cast<int>(threadIdx.x);
   const vec16 zero = {0u, 0u, 0u, 0u};
-  for (int row = begin; row < end; ++row) {
-    vec16* dst = a.recv_x + static_cast<size_t>(row) * a.row_vecs;
-    for (int v = tid; v < a.row_vecs; v += kPermuteThreads) dst[v] = zero;
-    if (a.recv_scales != nullptr)
-      for (int j = tid; j < a.num_scales; j += kPermuteThreads)
-        a.recv_scales[static_cast<size_t>(row) * a.num_scales + j] = 0.0f;
+  for (int row = begin + static_cast<int>(blockIdx.y); row < end; row += static_cast<int>(gridDim.y)) {
+    if (zero_payload) {
+      vec16* dst = a.recv_x + static_cast<size_t>(row) * a.row_vecs;
+      for (int v = tid; v < a.row_vecs; v += kPermuteThreads) __builtin_nontemporal_store(zero, dst + v);
+      if (a.recv_scales != nullptr)
+        for (int j = tid; j < a.num_scales; j += kPermuteThreads)
+          a.recv_scales[static_cast<size_t>(row) * a.num_scales + j] = 0.0f;
+    }
     if (tid == 0) {
       a.recv_src_map[row] = -1;
       if (a.recv_topk_idx != nullptr) a.recv_topk_idx[row] = -1;
@@ -580,8 +584,14 @@ hipError_t launch_pull_indices(const int* recv_src_map, int num_rows, int tokens
   return hipGetLastError();
 }
 
-hipError_t launch_pad_rows(const PermuteArgs& a, hipStream_t stream) {
-  hipLaunchKernelGGL(ep_pad_rows_kernel, dim3(a.num_experts), dim3(kPermuteThreads), 0, stream, a);
+hipError_t launch_pad_rows(const PermuteArgs& a, int expert_alignment, bool zero_payload, hipStream_t stream) {
+  // An expert has at most expert_alignment - 1 pad rows: one workgroup per possible pad row.
+  int per_expert = expert_alignment - 1;
+  if (per_expert < 1) return hipSuccess;
+  if (per_expert > 1024) per_expert = 1024;
+  if (!zero_payload) per_expert = 1;  // only the map entries: one workgroup per expert walks them
+  hipLaunchKernelGGL(ep_pad_rows_kernel, dim3(a.num_experts, per_expert), dim3(kPermuteThreads), 0, stream, a,
+                     zero_payload);
   return hipGetLastError();
 }
 

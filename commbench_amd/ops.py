@@ -24,6 +24,7 @@ from . import _lib
 MAX_RANKS = 8
 MAX_TOPK = 8
 MAX_EXPERTS = 1024
+KEEP_PAD_PAYLOAD = 1   # MI_EP_DISPATCH_KEEP_PAD_PAYLOAD
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -168,12 +169,14 @@ class Buffer:
     def dispatch(self, x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Tensor,
                  topk_weights: Optional[torch.Tensor], expert_alignment: int = 1,
                  num_channels: int = 0, handle: Optional[DispatchHandle] = None,
-                 capacity_rows: Optional[int] = None, rank_slot_base: Optional[int] = None):
+                 capacity_rows: Optional[int] = None, rank_slot_base: Optional[int] = None,
+                 zero_pads: bool = True):
         """Layout (unless `handle` is given) + permute into the expert-contiguous buffer.
 
         Returns (recv_x, recv_scales, recv_src_map, handle).  Buffers hold `capacity_rows` rows
         (default: the worst case T*K + E*(alignment-1), so no host sync is needed); rows at and
-        beyond handle.num_recv_rows() are unspecified.
+        beyond handle.num_recv_rows() are unspecified.  With expert_alignment > 1 the pad rows are
+        zero rows unless `zero_pads` is False (then only their map entries are written).
         """
         if handle is None:
             handle = self.dispatch_layout(topk_idx, expert_alignment, num_channels, rank_slot_base)
@@ -207,7 +210,8 @@ class Buffer:
             _ptr(handle.slot_rel), _ptr(handle.route_order), _ptr(handle.num_tokens_per_expert), T, K, E,
             handle.expert_alignment, row_bytes, num_scales, _ptr(recv_x), _ptr(recv_scales),
             _ptr(handle.recv_src_map), _ptr(handle.recv_topk_idx), _ptr(handle.recv_topk_weights),
-            _ptr(handle.slot_map), capacity_rows, _stream()), "mi_ep_dispatch")
+            _ptr(handle.slot_map), capacity_rows, 0 if zero_pads else KEEP_PAD_PAYLOAD, _stream()),
+            "mi_ep_dispatch")
         return recv_x, recv_scales, handle.recv_src_map, handle
 
 

@@ -30,6 +30,7 @@ extern "C" {
 
 /* Limits.  Ranks and top-k follow the reference's constructor checks
  * (example042_deepep_dispatch_layout/nv/empty_deepep_dispatch_layout.cu:43,46,96-107). */
+#define MI_EP_DISPATCH_KEEP_PAD_PAYLOAD 1
 #define MI_EP_MAX_RANKS 8
 #define MI_EP_MAX_TOPK 8
 #define MI_EP_MAX_EXPERTS 1024
@@ -142,7 +143,10 @@ size_t mi_ep_route_order_bytes(int num_tokens, int num_topk);
  *   slot_map     int32[num_tokens, num_topk]: absolute row of each route, -1 non-routes
  * Rows >= capacity_rows are never written.  With expert_alignment > 1 pad rows are
  * zero-filled; num_tokens_per_expert (from the layout call) locates them and may be
- * NULL when expert_alignment == 1.
+ * NULL when expert_alignment == 1.  flags: 0, or MI_EP_DISPATCH_KEEP_PAD_PAYLOAD to leave the
+ * payload and scales of pad rows untouched (their map entries are still written: source -1,
+ * expert -1, weight 0), for consumers that never look at what a pad row produces -- at
+ * alignment 128 the zero fill is a fifth of the copy.
  *   route_order  the layout call's table for the same topk_idx, or NULL.  The outputs are the
  *                same either way; with it, large shapes are copied in destination order
  *                (adjacent rows of recv_x written together, sources re-read from the L2 of the
@@ -154,7 +158,8 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
                    const int* route_order, const int* num_tokens_per_expert, int num_tokens, int num_topk,
                    int num_experts, int expert_alignment, int row_bytes, int num_scales,
                    void* recv_x, float* recv_scales, int* recv_src_map, int64_t* recv_topk_idx,
-                   float* recv_topk_weights, int* slot_map, int capacity_rows, void* stream);
+                   float* recv_topk_weights, int* slot_map, int capacity_rows, int flags,
+                   void* stream);
 
 /*
  * Dispatch de-duplicated by destination rank: the reference's own receive format (payload role

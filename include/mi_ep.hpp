@@ -183,7 +183,7 @@ class ExpertParallelBuffer {
                                h_.route_order, h_.num_tokens_per_expert, num_tokens, num_topk_, num_experts_,
                                h_.expert_alignment, row_bytes, num_scales, d_recv_x, d_recv_scales,
                                h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights, h_.slot_map,
-                               capacity_, stream));
+                               capacity_, /*flags=*/0, stream));
     return h_;
   }
 

@@ -67,7 +67,7 @@ def test_host_only_entry_points():
                                      None, None, 0, None, None, 0, None) == -22     # alignment 0
     assert lib.mi_ep_combine(None, 0, None, None, None, None, None, 4, 2, 12, None, None, None) == -22
     assert lib.mi_ep_dispatch(None, None, None, None, None, None, None, None, 4, 2, 8, 1, 24, 0,
-                              None, None, None, None, None, None, 0, None) == -22   # 24 % 16 != 0
+                              None, None, None, None, None, None, 0, 0, None) == -22   # 24 % 16 != 0
 
 
 def test_python_surface_rejects_bad_arguments_like_the_reference():

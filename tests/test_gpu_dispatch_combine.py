@@ -121,6 +121,31 @@ def test_alignment_pads_are_zero_rows(oracle, align):
     assert pads.any() and not gu.as_bytes(recv_x)[:off[-1]][pads].any()
 
 
+def test_pad_payload_can_be_left_alone(oracle):
+    """With the keep-pad-payload flag the pad rows keep what the buffer held; their map entries
+    and every real row are written as usual."""
+    rng = np.random.default_rng(6)
+    T, K, E, R, H, align = 600, 4, 32, 4, 128, 16
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    x_cpu = wl.bf16_normal(rng, T, H)
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    h = buf.dispatch_layout(torch.from_numpy(topk_np).to(gu.DEV), align)
+    # same layout handle, once with zero-filled pads and once with the pad payload left alone
+    filled = buf.dispatch(x_cpu.to(gu.DEV), None, torch.from_numpy(topk_np).to(gu.DEV), None, align, handle=h)
+    kept = buf.dispatch(x_cpu.to(gu.DEV), None, torch.from_numpy(topk_np).to(gu.DEV), None, align, handle=h,
+                        zero_pads=False)
+    torch.cuda.synchronize()
+    ref = oracle.full_path(topk_np, None, gu.as_bytes(x_cpu), None, E, R, align)
+    rows = int(ref["expert_offsets"][-1])
+    real = ref["recv_src_map"] >= 0
+    assert (~real).any()
+    for recv_x, _, src_map, hh in (filled, kept):
+        np.testing.assert_array_equal(src_map.cpu().numpy()[:rows], ref["recv_src_map"])
+        np.testing.assert_array_equal(hh.recv_topk_idx.cpu().numpy()[:rows], ref["recv_topk_idx"])
+        np.testing.assert_array_equal(gu.as_bytes(recv_x)[:rows][real], ref["recv_x"][real])
+    assert not gu.as_bytes(filled[0])[:rows][~real].any()
+
+
 @pytest.mark.parametrize("shape", [
     # T, K, E, R, row_bytes, num_scales
     (1, 1, 1, 1, 16, 0), (5, 3, 6, 2, 48, 1), (300, 8, 32, 4, 1024, 8), (300, 8, 32, 4, 1040, 0),

@@ -55,7 +55,7 @@ def test_graph_replays_match_eager(oracle, schedule):
         _lib.check(lib.mi_ep_dispatch(
             x.data_ptr(), None, topk.data_ptr(), w.data_ptr(), off.data_ptr(), slot_rel.data_ptr(),
             route_order.data_ptr(), per_expert.data_ptr(), T, K, E, 1, H * 2, 0, recv_x.data_ptr(), None, src_map.data_ptr(),
-            recv_idx.data_ptr(), recv_w.data_ptr(), slot_map.data_ptr(), cap, stream), "dispatch")
+            recv_idx.data_ptr(), recv_w.data_ptr(), slot_map.data_ptr(), cap, 0, stream), "dispatch")
         _lib.check(lib.mi_ep_combine(
             recv_x.data_ptr(), cap, slot_map.data_ptr(), w.data_ptr(), None, None, None, T, K, H,
             out.data_ptr(), None, stream), "combine")
