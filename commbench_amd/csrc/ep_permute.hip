@@ -1,5 +1,11 @@
 // Permute (dispatch payload) kernels for gfx950.
 //
+// Three copies with the same outputs but different orders and formats:
+//   ep_permute_tiles_kernel   destination order, for long rows on large batches (further down)
+//   ep_permute_kernel         token order, everything else
+//   ep_permute_ranks_kernel   one row per (token, destination rank), the reference's own format
+// plus the pad-row fill, the pull-mode gathers and the bandwidth yardsticks.
+//
 // ep_permute_kernel: each wavefront owns (token, batch): one batch is up to
 // kBatchVecs * 64 consecutive 16-byte vectors of the token's row (1 KiB as launched).  The wave reads
 // its batch once into registers and stores it to every row the token was routed
@@ -115,7 +121,7 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
 // accelerator die j % 8 (workgroup b is dispatched to die b % 8: read back from the XCC_ID
 // register, every workgroup of a 3-D grid sat on die (linear id) % 8) and a tile's 256 rows
 // fit that die's 4 MiB L2, so the repeats never leave the die.  A workgroup copies
-// kPushWaves KiB of one route's row; part 0 also writes the row's side data.
+// kPushWaves * kVecs KiB of one route's row; part 0 also writes the row's side data.
 // Launched as a 3-D grid (x = part of the row * 8 + die, y = entry of the tile's list, z = round
 // of eight tiles) so that no index needs a division: a wave moves only 1 KiB, which leaves it
 // a budget of about a hundred vector instructions before instruction issue, not HBM, sets the pace.
