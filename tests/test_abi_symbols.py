@@ -56,6 +56,19 @@ def test_host_only_entry_points():
     assert lib.mi_ep_dispatch_schedule_for(8192, 2, 1024, 14336) == 1    # half a row per tile and expert
     assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 16384) == 1     # a tile's rows exceed L2
     assert lib.mi_ep_dispatch_schedule_for(8192, 8, 256, 100) == -22
+    # the per-rank format, the pull form and the host twins check their arguments before any launch
+    assert lib.mi_ep_dispatch_ranks(None, None, None, None, None, 0, None, None, 4, 2, 3, 8, 32, 0, 0, 0,
+                                    None, None, None, None, None, None, None, None, 0, None) == -22   # 8 % 3
+    assert lib.mi_ep_dispatch_ranks(None, None, None, None, None, 0, None, None, 4, 2, 2, 8, 24, 0, 0, 0,
+                                    None, None, None, None, None, None, None, None, 0, None) == -22   # 24 % 16
+    assert lib.mi_ep_combine_rank_weights(None, None, 4, 9, 0, None, None) == -22                    # 9 slots
+    assert lib.mi_ep_dispatch_cached(None, None, None, 4, 4, 24, 0, None, None, None, 0, None) == -22
+    assert lib.mi_ep_dispatch(None, None, None, None, None, None, None, None, 4, 2, 8, 1, 32, 0,
+                              None, None, None, None, None, None, 0, 2, None) == -22   # null tables (and an unknown flag)
+    assert lib.mi_ep_host_get_dispatch_layout(None, None, None, None, None, 4, 2, 2, 8) == -22
+    assert lib.mi_ep_host_dispatch(None, None, None, None, 4, 2, 2, 8, 1, 24, 0, None, None, None, None,
+                                   None, None, None, None, None, None, 0) == -22
+    assert lib.mi_ep_host_combine(None, 0, None, None, None, None, 4, 2, 12, None) == -22
     assert lib.mi_ep_workspace_bytes(8192, 8, 256, 9) == 0       # more than 8 ranks
     assert lib.mi_ep_workspace_bytes(8192, 9, 256, 8) == 0       # more than 8 slots
     assert lib.mi_ep_workspace_bytes(8192, 8, 250, 8) == 0       # experts not divisible by ranks
