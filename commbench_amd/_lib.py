@@ -26,6 +26,10 @@ SIGNATURES = {
     "mi_ep_route_order_bytes": (_size, [_int, _int]),
     "mi_ep_dispatch": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int,
                               _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
+    "mi_ep_dispatch_strided_scales": (_int, [_vp, _vp, ctypes.c_longlong, ctypes.c_longlong, _vp, _vp, _vp, _vp, _vp,
+                                             _vp, _int, _int, _int, _int, _int, _int, _vp, _vp,
+                                             ctypes.c_longlong, ctypes.c_longlong, _vp, _vp, _vp, _vp, _int, _int,
+                                             _vp]),
     "mi_ep_dispatch_ranks": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _int, _int, _int, _int, _int,
                                     _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
     "mi_ep_combine_rank_weights": (_int, [_vp, _vp, _int, _int, _int, _vp, _vp]),

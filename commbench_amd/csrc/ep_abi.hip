@@ -190,11 +190,13 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
   return status_of(launch_layout_fused(a, s));
 }
 
-int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
+int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long long x_scales_token_stride,
+                                  long long x_scales_hidden_stride, const int64_t* topk_idx,
                    const float* topk_weights, const int* expert_offsets, const int* slot_rel,
                    const int* route_order, const int* num_tokens_per_expert, int num_tokens, int num_topk,
                    int num_experts, int expert_alignment, int row_bytes, int num_scales,
-                   void* recv_x, float* recv_scales, int* recv_src_map, int64_t* recv_topk_idx,
+                   void* recv_x, float* recv_scales, long long recv_scales_token_stride,
+                   long long recv_scales_hidden_stride, int* recv_src_map, int64_t* recv_topk_idx,
                    float* recv_topk_weights, int* slot_map, int capacity_rows, int flags,
                    void* stream) {
   if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK) return MI_EP_EINVAL;
@@ -210,6 +212,9 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
   if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
   if (expert_alignment > 1 && num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
   if ((flags & ~MI_EP_DISPATCH_KEEP_PAD_PAYLOAD) != 0) return MI_EP_EINVAL;
+  if (num_scales > 0 && (x_scales_token_stride < 0 || x_scales_hidden_stride < 0 ||
+                         recv_scales_token_stride < 0 || recv_scales_hidden_stride < 0))
+    return MI_EP_EINVAL;
 
   PermuteArgs a{};
   a.x = static_cast<const vec16*>(x);
@@ -232,10 +237,28 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
   a.row_vecs = row_bytes / 16;
   a.num_scales = num_scales;
   a.capacity_rows = capacity_rows;
+  a.xs_token_stride = x_scales_token_stride;
+  a.xs_hidden_stride = x_scales_hidden_stride;
+  a.rs_token_stride = recv_scales_token_stride;
+  a.rs_hidden_stride = recv_scales_hidden_stride;
   hipStream_t s = as_stream(stream);
   hipError_t e = launch_permute(a, g_permute_schedule.load(std::memory_order_relaxed), s);
   if (e == hipSuccess && expert_alignment > 1) e = launch_pad_rows(a, expert_alignment, (flags & MI_EP_DISPATCH_KEEP_PAD_PAYLOAD) == 0, s);
   return status_of(e);
+}
+
+int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
+                   const float* topk_weights, const int* expert_offsets, const int* slot_rel,
+                   const int* route_order, const int* num_tokens_per_expert, int num_tokens, int num_topk,
+                   int num_experts, int expert_alignment, int row_bytes, int num_scales,
+                   void* recv_x, float* recv_scales, int* recv_src_map, int64_t* recv_topk_idx,
+                   float* recv_topk_weights, int* slot_map, int capacity_rows, int flags,
+                   void* stream) {
+  return mi_ep_dispatch_strided_scales(x, x_scales, num_scales, 1, topk_idx, topk_weights, expert_offsets,
+                                       slot_rel, route_order, num_tokens_per_expert, num_tokens, num_topk,
+                                       num_experts, expert_alignment, row_bytes, num_scales, recv_x,
+                                       recv_scales, num_scales, 1, recv_src_map, recv_topk_idx,
+                                       recv_topk_weights, slot_map, capacity_rows, flags, stream);
 }
 
 int mi_ep_dispatch_ranks(const void* x, const float* x_scales, const int64_t* topk_idx,

@@ -87,6 +87,10 @@ struct PermuteArgs {
   int row_vecs;  // 16-byte vectors per row
   int num_scales;
   int capacity_rows;
+  // Scale factors are addressed as [row * token_stride + j * hidden_stride], in 4-byte elements
+  // (sf_token_stride / sf_hidden_stride of the reference's dispatch, example080 .cu:40).
+  long long xs_token_stride, xs_hidden_stride;
+  long long rs_token_stride, rs_hidden_stride;
 };
 
 // Which copy kernel serves mi_ep_dispatch: chosen by shape, or forced (tests, measurements).

@@ -84,10 +84,12 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
 
   if (batch == 0 && a.recv_scales != nullptr) {
     for (int j = lane; j < a.num_scales; j += kWave) {
-      const float s = a.x_scales[static_cast<size_t>(token) * a.num_scales + j];
+      const float s = a.x_scales[static_cast<size_t>(token) * a.xs_token_stride +
+                                 static_cast<size_t>(j) * a.xs_hidden_stride];
       for (int k = 0; k < K; ++k) {
         const int row = wave_read(slot, k);
-        if (row >= 0) a.recv_scales[static_cast<size_t>(row) * a.num_scales + j] = s;
+        if (row >= 0)
+          a.recv_scales[static_cast<size_t>(row) * a.rs_token_stride + static_cast<size_t>(j) * a.rs_hidden_stride] = s;
       }
     }
   }
@@ -198,8 +200,8 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
     }
     if (slot >= 0 && a.recv_scales != nullptr)
       for (int j = lane; j < a.num_scales; j += kWave)
-        a.recv_scales[static_cast<size_t>(slot) * a.num_scales + j] =
-            a.x_scales[static_cast<size_t>(token) * a.num_scales + j];
+        a.recv_scales[static_cast<size_t>(slot) * a.rs_token_stride + static_cast<size_t>(j) * a.rs_hidden_stride] =
+            a.x_scales[static_cast<size_t>(token) * a.xs_token_stride + static_cast<size_t>(j) * a.xs_hidden_stride];
   }
   if (slot >= 0) {
 #pragma unroll
@@ -342,7 +344,7 @@ __global__ __launch_bounds__(kPermuteThreads) void ep_pad_rows_kernel(const Perm
       for (int v = tid; v < a.row_vecs; v += kPermuteThreads) __builtin_nontemporal_store(zero, dst + v);
       if (a.recv_scales != nullptr)
         for (int j = tid; j < a.num_scales; j += kPermuteThreads)
-          a.recv_scales[static_cast<size_t>(row) * a.num_scales + j] = 0.0f;
+          a.recv_scales[static_cast<size_t>(row) * a.rs_token_stride + static_cast<size_t>(j) * a.rs_hidden_stride] = 0.0f;
     }
     if (tid == 0) {
       a.recv_src_map[row] = -1;

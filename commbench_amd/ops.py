@@ -170,13 +170,16 @@ class Buffer:
                  topk_weights: Optional[torch.Tensor], expert_alignment: int = 1,
                  num_channels: int = 0, handle: Optional[DispatchHandle] = None,
                  capacity_rows: Optional[int] = None, rank_slot_base: Optional[int] = None,
-                 zero_pads: bool = True):
+                 zero_pads: bool = True, column_major_recv_scales: bool = False):
         """Layout (unless `handle` is given) + permute into the expert-contiguous buffer.
 
         Returns (recv_x, recv_scales, recv_src_map, handle).  Buffers hold `capacity_rows` rows
         (default: the worst case T*K + E*(alignment-1), so no host sync is needed); rows at and
         beyond handle.num_recv_rows() are unspecified.  With expert_alignment > 1 the pad rows are
         zero rows unless `zero_pads` is False (then only their map entries are written).
+        `scales` may be any 2-D float32 view (row- or column-major, padded); with
+        `column_major_recv_scales` the returned recv_scales is a [capacity, S] view of a [S, capacity]
+        allocation, the layout the reference's TMA-aligned scale tensors have.
         """
         if handle is None:
             handle = self.dispatch_layout(topk_idx, expert_alignment, num_channels, rank_slot_base)
@@ -187,8 +190,8 @@ class Buffer:
         _require(row_bytes % 16 == 0, "row size must be a multiple of 16 bytes")
         num_scales = 0
         if scales is not None:
-            _require(scales.dtype == torch.float32 and scales.dim() == 2 and scales.is_contiguous()
-                     and scales.shape[0] == T, "scales must be contiguous float32 [num_tokens, S]")
+            _require(scales.dtype == torch.float32 and scales.dim() == 2 and scales.shape[0] == T
+                     and min(scales.stride()) >= 0, "scales must be a float32 [num_tokens, S] tensor or view")
             num_scales = scales.shape[1]
         if topk_weights is not None:
             _require(topk_weights.dtype == torch.float32 and topk_weights.is_contiguous()
@@ -198,20 +201,25 @@ class Buffer:
             capacity_rows = T * K + E * (handle.expert_alignment - 1)
         dev = x.device
         recv_x = torch.empty((capacity_rows, x.shape[1]), dtype=x.dtype, device=dev)
-        recv_scales = (torch.empty((capacity_rows, num_scales), dtype=torch.float32, device=dev)
-                       if scales is not None else None)
+        recv_scales = None
+        if scales is not None and column_major_recv_scales:
+            recv_scales = torch.empty((num_scales, capacity_rows), dtype=torch.float32, device=dev).t()
+        elif scales is not None:
+            recv_scales = torch.empty((capacity_rows, num_scales), dtype=torch.float32, device=dev)
+        xs_strides = scales.stride() if scales is not None else (0, 0)
+        rs_strides = recv_scales.stride() if recv_scales is not None else (0, 0)
         handle.recv_src_map = torch.empty(capacity_rows, dtype=torch.int32, device=dev)
         handle.recv_topk_idx = torch.empty(capacity_rows, dtype=torch.int64, device=dev)
         handle.recv_topk_weights = torch.empty(capacity_rows, dtype=torch.float32, device=dev)
         handle.slot_map = torch.empty((T, K), dtype=torch.int32, device=dev)
         lib = _lib.load()
-        _lib.check(lib.mi_ep_dispatch(
-            _ptr(x), _ptr(scales), _ptr(topk_idx), _ptr(topk_weights), _ptr(handle.expert_offsets),
-            _ptr(handle.slot_rel), _ptr(handle.route_order), _ptr(handle.num_tokens_per_expert), T, K, E,
-            handle.expert_alignment, row_bytes, num_scales, _ptr(recv_x), _ptr(recv_scales),
-            _ptr(handle.recv_src_map), _ptr(handle.recv_topk_idx), _ptr(handle.recv_topk_weights),
-            _ptr(handle.slot_map), capacity_rows, 0 if zero_pads else KEEP_PAD_PAYLOAD, _stream()),
-            "mi_ep_dispatch")
+        _lib.check(lib.mi_ep_dispatch_strided_scales(
+            _ptr(x), _ptr(scales), xs_strides[0], xs_strides[1], _ptr(topk_idx), _ptr(topk_weights),
+            _ptr(handle.expert_offsets), _ptr(handle.slot_rel), _ptr(handle.route_order),
+            _ptr(handle.num_tokens_per_expert), T, K, E, handle.expert_alignment, row_bytes, num_scales,
+            _ptr(recv_x), _ptr(recv_scales), rs_strides[0], rs_strides[1], _ptr(handle.recv_src_map),
+            _ptr(handle.recv_topk_idx), _ptr(handle.recv_topk_weights), _ptr(handle.slot_map), capacity_rows, 0 if zero_pads else KEEP_PAD_PAYLOAD, _stream()),
+            "mi_ep_dispatch_strided_scales")
         return recv_x, recv_scales, handle.recv_src_map, handle
 
 

@@ -162,6 +162,25 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
                    void* stream);
 
 /*
+ * The same call with the scale factors addressed through strides, as the reference's dispatch
+ * takes them (sf_token_stride, sf_hidden_stride, example080 .cu:40; recv_sf_token_stride,
+ * recv_sf_hidden_stride, example081 .cu:31): element j of row r sits at
+ * base[r * token_stride + j * hidden_stride], strides counted in 4-byte elements (a float, or
+ * a pack of four 8-bit exponents: the copy does not look inside).  mi_ep_dispatch is this call
+ * with strides (num_scales, 1) on both sides.  Column-major scale tensors, which the reference's
+ * TMA-aligned layouts use, are (1, padded row count).
+ */
+int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long long x_scales_token_stride,
+                                  long long x_scales_hidden_stride, const int64_t* topk_idx,
+                                  const float* topk_weights, const int* expert_offsets, const int* slot_rel,
+                                  const int* route_order, const int* num_tokens_per_expert, int num_tokens,
+                                  int num_topk, int num_experts, int expert_alignment, int row_bytes,
+                                  int num_scales, void* recv_x, float* recv_scales,
+                                  long long recv_scales_token_stride, long long recv_scales_hidden_stride,
+                                  int* recv_src_map, int64_t* recv_topk_idx, float* recv_topk_weights,
+                                  int* slot_map, int capacity_rows, int flags, void* stream);
+
+/*
  * Dispatch de-duplicated by destination rank: the reference's own receive format (payload role
  * of dispatch_impl, example080_deepep_jit_dispatch_payload/nv/empty_deepep_jit_dispatch_payload.cu:31-44,
  * 241-256, then dispatch_copy_epilogue_impl without expansion,

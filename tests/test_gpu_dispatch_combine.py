@@ -121,6 +121,38 @@ def test_alignment_pads_are_zero_rows(oracle, align):
     assert pads.any() and not gu.as_bytes(recv_x)[:off[-1]][pads].any()
 
 
+@pytest.mark.parametrize("schedule", [gu.SCHEDULE_BY_TOKEN, gu.SCHEDULE_BY_DESTINATION])
+def test_scale_factors_through_strides(oracle, schedule):
+    """Scale factors in a column-major, padded tensor on the way in and column-major on the way out
+    (the reference addresses them through token and hidden strides, example080 .cu:40)."""
+    from commbench_amd import _lib
+    rng = np.random.default_rng(40)
+    T, K, E, R, H, align = 777, 8, 32, 8, 1024, 16
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    topk_np[rng.random((T, K)) < 0.05] = -1
+    xq, scales_cpu = wl.quantize_fp8_blockwise(wl.bf16_normal(rng, T, H))
+    S = scales_cpu.shape[1]
+    padded = torch.full((S, T + 19), -7.0, dtype=torch.float32, device=gu.DEV)   # [S, T padded], column-major view
+    padded[:, :T] = scales_cpu.t().to(gu.DEV)
+    scales_view = padded[:, :T].t()
+    assert not scales_view.is_contiguous() and scales_view.stride() == (1, T + 19)
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    lib = _lib.load()
+    assert lib.mi_ep_set_dispatch_schedule(schedule) == 0
+    try:
+        recv_x, recv_scales, _, h = buf.dispatch(xq.to(gu.DEV), scales_view, torch.from_numpy(topk_np).to(gu.DEV),
+                                                 None, expert_alignment=align, column_major_recv_scales=True)
+        torch.cuda.synchronize()
+    finally:
+        assert lib.mi_ep_set_dispatch_schedule(gu.SCHEDULE_AUTO) == 0
+    ref = oracle.full_path(topk_np, None, gu.as_bytes(xq), scales_cpu.numpy(), E, R, align)
+    rows = int(ref["expert_offsets"][-1])
+    assert recv_scales.stride()[0] == 1                                    # column-major as asked
+    np.testing.assert_array_equal(gu.as_bytes(recv_x)[:rows], ref["recv_x"])
+    np.testing.assert_array_equal(recv_scales.cpu().numpy()[:rows].view(np.uint32), ref["recv_scales"].view(np.uint32))
+    assert (padded[:, T:] == -7.0).all()                                   # the padding was not touched
+
+
 def test_pad_payload_can_be_left_alone(oracle):
     """With the keep-pad-payload flag the pad rows keep what the buffer held; their map entries
     and every real row are written as usual."""
