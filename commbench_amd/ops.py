@@ -10,6 +10,11 @@ split into `num_ranks` partitions:
     dispatch(x, scales, topk_idx, topk_weights, ...)
         -> (recv_x, recv_scales, recv_src_map, handle)
     combine(y, slot_map | handle, topk_weights) -> combined_x
+    dispatch_ranks(buffer, x, scales, topk_idx, topk_weights, ...)       the reference's own receive
+        -> (recv_x, recv_topk_idx, recv_topk_weights, handle)            format: one row per token
+    combine_ranks(y, handle, recv_topk_weights) -> combined_x[, weights]  and destination rank
+    dispatch_cached / pull_indices                                        pull form from a source map
+    host_get_dispatch_layout / host_dispatch / host_combine               numpy in, numpy out
 
 torch is used for device memory and streams only; all arithmetic runs in the HIP kernels of
 libmi_ep.so.  Nothing here falls back to torch ops or to the CPU.
