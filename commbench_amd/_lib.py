@@ -23,6 +23,8 @@ SIGNATURES = {
     "mi_ep_dispatch_schedule_for": (_int, [_int, _int, _int, _int]),
     "mi_ep_dispatch_layout": (_int, [_vp, _int, _int, _int, _int, _int, _int,
                                      _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _size, _vp]),
+    "mi_ep_dispatch_layout_static": (_int, [_vp, _int, _int, _int, _int, _int, _int,
+                                            _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp]),
     "mi_ep_route_order_bytes": (_size, [_int, _int]),
     "mi_ep_dispatch": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int,
                               _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),

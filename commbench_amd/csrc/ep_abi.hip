@@ -38,6 +38,107 @@ constexpr uint32_t kSpinLimit = 1u << 22;
 std::atomic<uint32_t> g_spin_limit{kSpinLimit};  // only ever changed by the test hook
 std::atomic<int> g_permute_schedule{kPermuteAuto};
 
+// Argument checks and launch shared by mi_ep_dispatch_layout (caller's workspace) and
+// mi_ep_dispatch_layout_static (the library's static scratch); `workspace_words` is the number of
+// status words behind the workspace header.
+int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
+                       int num_experts, int expert_alignment, int num_channels,
+                       int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
+                       int* expert_offsets, int* psum_rank_rows, int* channel_prefix_matrix,
+                       int* slot_rel, int* rank_slot_idx, int rank_slot_base, int* route_order,
+                       void* workspace, size_t workspace_bytes, int too_small_code,
+                       int* timeout_report, void* stream) {
+  if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
+  if (expert_alignment < 1) return MI_EP_EINVAL;
+  if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
+  if (channel_prefix_matrix != nullptr && (num_channels < 1 || num_channels > 4096)) return MI_EP_EINVAL;
+  if (psum_rank_rows != nullptr && expert_offsets == nullptr) return MI_EP_EINVAL;
+  // Padded totals must stay inside int32.
+  if ((static_cast<long long>(num_tokens) * num_topk +
+       static_cast<long long>(num_experts) * (expert_alignment - 1)) >= (1LL << 31))
+    return MI_EP_EINVAL;
+  hipStream_t s = as_stream(stream);
+
+  if (num_tokens == 0) {
+    // Nothing to scan: every output is zero.
+    hipError_t e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_rank), num_ranks, 0u, s);
+    if (e == hipSuccess)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_expert), num_experts, 0u, s);
+    if (e == hipSuccess && expert_offsets != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(expert_offsets), num_experts + 1, 0u, s);
+    if (e == hipSuccess && psum_rank_rows != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(psum_rank_rows), num_ranks, 0u, s);
+    if (e == hipSuccess && channel_prefix_matrix != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(channel_prefix_matrix),
+                          static_cast<size_t>(num_ranks) * num_channels, 0u, s);
+    return status_of(e);
+  }
+
+  if (topk_idx == nullptr || is_token_in_rank == nullptr || workspace == nullptr) return MI_EP_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
+  if (!aligned16(route_order)) return MI_EP_EINVAL;
+  if (workspace_bytes < mi_ep_workspace_bytes(num_tokens, num_topk, num_experts, num_ranks))
+    return too_small_code;
+
+  LayoutArgs a{};
+  a.topk_idx = topk_idx;
+  a.num_tokens_per_rank = num_tokens_per_rank;
+  a.num_tokens_per_expert = num_tokens_per_expert;
+  a.is_token_in_rank = reinterpret_cast<uint8_t*>(is_token_in_rank);
+  a.expert_offsets = expert_offsets;
+  a.psum_rank_rows = psum_rank_rows;
+  a.channel_prefix_matrix = channel_prefix_matrix;
+  a.slot_rel = slot_rel;
+  a.rank_slot_idx = rank_slot_idx;
+  a.rank_slot_base = rank_slot_base;
+  a.route_order = route_order;
+  a.ws = static_cast<LayoutWorkspace*>(workspace);
+  a.timeout_report = timeout_report;
+  a.num_tokens = num_tokens;
+  a.num_topk = num_topk;
+  a.num_ranks = num_ranks;
+  a.num_experts = num_experts;
+  a.experts_per_rank = num_experts / num_ranks;
+  a.expert_alignment = expert_alignment;
+  a.num_channels = num_channels;
+  a.num_tiles = num_tiles_for(num_tokens);
+  a.expert_bits = 1;
+  while ((1 << a.expert_bits) < num_experts) ++a.expert_bits;
+  a.inv_topk = ((1u << 19) + num_topk - 1) / num_topk;
+  a.inv_experts_per_rank = ((1u << 22) + a.experts_per_rank - 1) / a.experts_per_rank;
+  a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+  return status_of(launch_layout_fused(a, s));
+}
+
+// ---- scratch of the allocation-free layout entry point ------------------------------------
+// One copy per GPU, held until the process ends: the layout workspace (256-byte header + status
+// words) for shapes up to MI_EP_STATIC_LAYOUT_STATUS_WORDS status words.  `scratch` is a host-side
+// stand-in here; kernels get the device address resolved below.
+constexpr size_t kStaticStatusWords = MI_EP_STATIC_LAYOUT_STATUS_WORDS;
+constexpr size_t kStaticScratchBytes = sizeof(LayoutWorkspace) + kStaticStatusWords * sizeof(uint64_t);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+// Device address of `scratch` per device ordinal: resolved on the first call on that device,
+// read-only afterwards (every resolver stores the same value).
+std::atomic<void*> g_scratch_address[kMaxDevices];
+
+int static_scratch_of_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= kMaxDevices) return MI_EP_EINVAL;
+  void* p = g_scratch_address[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (p == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+    g_scratch_address[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return MI_EP_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -49,6 +150,7 @@ const char* mi_ep_strerror(int code) {
     case MI_EP_OK: return "ok";
     case MI_EP_EINVAL: return "invalid argument";
     case MI_EP_ENOSPC: return "workspace too small";
+    case MI_EP_E2BIG: return "shape exceeds the static scratch of the allocation-free entry point";
     case MI_EP_ETIMEDOUT: return "device-side wait timed out";
     default: break;
   }
@@ -129,65 +231,35 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
                           int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
                           int rank_slot_base, int* route_order, void* workspace,
                           size_t workspace_bytes, void* stream) {
+  return dispatch_layout_on(topk_idx, num_tokens, num_topk, num_ranks, num_experts, expert_alignment,
+                            num_channels, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank,
+                            expert_offsets, psum_rank_rows, channel_prefix_matrix, slot_rel, rank_slot_idx,
+                            rank_slot_base, route_order, workspace, workspace_bytes, MI_EP_ENOSPC, nullptr,
+                            stream);
+}
+
+int mi_ep_dispatch_layout_static(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
+                                 int num_experts, int expert_alignment, int num_channels,
+                                 int* num_tokens_per_rank, int* num_tokens_per_expert,
+                                 bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
+                                 int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
+                                 int rank_slot_base, int* route_order, int* timeout_report, void* stream) {
+  // The shape check comes first so that an oversized request is refused before anything else.
   if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
-  if (expert_alignment < 1) return MI_EP_EINVAL;
-  if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
-  if (channel_prefix_matrix != nullptr && (num_channels < 1 || num_channels > 4096)) return MI_EP_EINVAL;
-  if (psum_rank_rows != nullptr && expert_offsets == nullptr) return MI_EP_EINVAL;
-  // Padded totals must stay inside int32.
-  if ((static_cast<long long>(num_tokens) * num_topk +
-       static_cast<long long>(num_experts) * (expert_alignment - 1)) >= (1LL << 31))
-    return MI_EP_EINVAL;
-  hipStream_t s = as_stream(stream);
-
-  if (num_tokens == 0) {
-    // Nothing to scan: every output is zero.
-    hipError_t e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_rank), num_ranks, 0u, s);
-    if (e == hipSuccess)
-      e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_expert), num_experts, 0u, s);
-    if (e == hipSuccess && expert_offsets != nullptr)
-      e = launch_fill_u32(reinterpret_cast<uint32_t*>(expert_offsets), num_experts + 1, 0u, s);
-    if (e == hipSuccess && psum_rank_rows != nullptr)
-      e = launch_fill_u32(reinterpret_cast<uint32_t*>(psum_rank_rows), num_ranks, 0u, s);
-    if (e == hipSuccess && channel_prefix_matrix != nullptr)
-      e = launch_fill_u32(reinterpret_cast<uint32_t*>(channel_prefix_matrix),
-                          static_cast<size_t>(num_ranks) * num_channels, 0u, s);
-    return status_of(e);
-  }
-
-  if (topk_idx == nullptr || is_token_in_rank == nullptr || workspace == nullptr) return MI_EP_EINVAL;
-  if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
-  if (!aligned16(route_order)) return MI_EP_EINVAL;
-  if (workspace_bytes < mi_ep_workspace_bytes(num_tokens, num_topk, num_experts, num_ranks))
-    return MI_EP_ENOSPC;
-
-  LayoutArgs a{};
-  a.topk_idx = topk_idx;
-  a.num_tokens_per_rank = num_tokens_per_rank;
-  a.num_tokens_per_expert = num_tokens_per_expert;
-  a.is_token_in_rank = reinterpret_cast<uint8_t*>(is_token_in_rank);
-  a.expert_offsets = expert_offsets;
-  a.psum_rank_rows = psum_rank_rows;
-  a.channel_prefix_matrix = channel_prefix_matrix;
-  a.slot_rel = slot_rel;
-  a.rank_slot_idx = rank_slot_idx;
-  a.rank_slot_base = rank_slot_base;
-  a.route_order = route_order;
-  a.ws = static_cast<LayoutWorkspace*>(workspace);
-  a.num_tokens = num_tokens;
-  a.num_topk = num_topk;
-  a.num_ranks = num_ranks;
-  a.num_experts = num_experts;
-  a.experts_per_rank = num_experts / num_ranks;
-  a.expert_alignment = expert_alignment;
-  a.num_channels = num_channels;
-  a.num_tiles = num_tiles_for(num_tokens);
-  a.expert_bits = 1;
-  while ((1 << a.expert_bits) < num_experts) ++a.expert_bits;
-  a.inv_topk = ((1u << 19) + num_topk - 1) / num_topk;
-  a.inv_experts_per_rank = ((1u << 22) + a.experts_per_rank - 1) / a.experts_per_rank;
-  a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
-  return status_of(launch_layout_fused(a, s));
+  if (static_cast<size_t>(num_tiles_for(num_tokens)) * static_cast<size_t>(num_experts + num_ranks) >
+      kStaticStatusWords)
+    return MI_EP_E2BIG;
+  void* ws = nullptr;
+  const int rc = static_scratch_of_current_device(&ws);
+  if (rc != MI_EP_OK) return rc;
+  // Nothing needs clearing between calls: the scratch starts zeroed when the code object is
+  // loaded (an initialised workspace), and every launch leaves the ticket word ready for the
+  // next and tags its status words with a fresh generation.
+  return dispatch_layout_on(topk_idx, num_tokens, num_topk, num_ranks, num_experts, expert_alignment,
+                            num_channels, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank,
+                            expert_offsets, psum_rank_rows, channel_prefix_matrix, slot_rel, rank_slot_idx,
+                            rank_slot_base, route_order, ws, kStaticScratchBytes, MI_EP_E2BIG,
+                            timeout_report, stream);
 }
 
 int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long long x_scales_token_stride,

@@ -43,6 +43,7 @@ struct LayoutArgs {
   int* rank_slot_idx;
   int* route_order;  // [num_tiles * kTileTokens * K][4] or null
   LayoutWorkspace* ws;
+  int* timeout_report;  // null, or a device word that receives MI_EP_ETIMEDOUT when a bounded wait expires
   int num_tokens;
   int num_topk;
   int num_ranks;

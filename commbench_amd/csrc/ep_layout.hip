@@ -39,6 +39,7 @@ constexpr uint32_t kFlagAggregate = 1;
 constexpr uint32_t kFlagPrefix = 2;
 constexpr uint32_t kGenMask = 0x3fffffffu;
 constexpr int kLookbackWindow = 32;
+constexpr int kTimedOutCode = -110;  // MI_EP_ETIMEDOUT of the C ABI
 constexpr int kCountsThreads = 1024;  // the counts-only kernel: one token per thread, 16 waves
 
 __device__ __forceinline__ uint64_t pack_status(uint32_t flag, uint32_t gen, uint32_t value) {
@@ -274,6 +275,8 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
         if (stalled) {
           if (++spins >= a.spin_limit) {
             __hip_atomic_store(&a.ws->timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (a.timeout_report != nullptr)
+              __hip_atomic_store(a.timeout_report, kTimedOutCode, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             break;
           }
           __builtin_amdgcn_s_sleep(2);

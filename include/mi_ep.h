@@ -27,6 +27,7 @@ extern "C" {
 #define MI_EP_EINVAL (-22)    /* argument out of range or NULL where required */
 #define MI_EP_ENOSPC (-28)    /* workspace too small */
 #define MI_EP_ETIMEDOUT (-110) /* device-side bounded wait expired (mi_ep_workspace_status) */
+#define MI_EP_E2BIG (-7)      /* shape exceeds the static scratch of mi_ep_dispatch_layout_static */
 
 /* Limits.  Ranks and top-k follow the reference's constructor checks
  * (example042_deepep_dispatch_layout/nv/empty_deepep_dispatch_layout.cu:43,46,96-107). */
@@ -121,6 +122,32 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
                           int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
                           int rank_slot_base, int* route_order, void* workspace,
                           size_t workspace_bytes, void* stream);
+/*
+ * mi_ep_dispatch_layout without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory or carry a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The look-back status words live in a static device array inside the library (2 MiB + 256 bytes
+ * on every GPU the library runs on, held until the process ends).  Same arguments, outputs and
+ * results as mi_ep_dispatch_layout.
+ *   limit    ceil(num_tokens / 256) * (num_experts + num_ranks) <= MI_EP_STATIC_LAYOUT_STATUS_WORDS
+ *            (254 000 tokens at 256 experts, 65 000 at 1024); beyond it the call returns
+ *            MI_EP_E2BIG and launches nothing.
+ *   timeout_report  NULL, or one int32 of device memory that the caller has set to 0: receives
+ *            MI_EP_ETIMEDOUT if a bounded device-side wait of this launch expires (the outputs are
+ *            then unspecified); never written otherwise.
+ * Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race and give unspecified results; calls ordered on one stream, or
+ * otherwise serialised, are safe back to back whatever their shapes.  The first call on a device
+ * resolves the array's address (hipGetSymbolAddress, which may load the code object): make it
+ * outside graph capture.  Calls hipMalloc / hipFree never.
+ */
+#define MI_EP_STATIC_LAYOUT_STATUS_WORDS 262144
+int mi_ep_dispatch_layout_static(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
+                                 int num_experts, int expert_alignment, int num_channels,
+                                 int* num_tokens_per_rank, int* num_tokens_per_expert,
+                                 bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
+                                 int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
+                                 int rank_slot_base, int* route_order, int* timeout_report, void* stream);
 /* Bytes of route_order for this shape. */
 size_t mi_ep_route_order_bytes(int num_tokens, int num_topk);
 

@@ -1,0 +1,101 @@
+"""GPU parity of the allocation-free layout entry point (mi_ep_dispatch_layout_static) against
+mi_ep_dispatch_layout, through the C ABI: every output bit-exact, on calls in a row that share
+the library's static scratch, the later ones with smaller inputs."""
+import numpy as np
+import pytest
+import torch
+
+from commbench_amd import _lib
+from commbench_amd import workloads as wl
+
+from . import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+
+STATUS_WORDS = 262144      # MI_EP_STATIC_LAYOUT_STATUS_WORDS
+E2BIG = -7
+
+
+class LayoutOutputs:
+    """One set of output buffers for either entry point, pre-filled with a pattern."""
+
+    def __init__(self, T, K, R, E, channels, lib):
+        i32 = dict(dtype=torch.int32, device=gu.DEV)
+        self.per_rank = torch.full((R,), -3, **i32)
+        self.per_expert = torch.full((E,), -3, **i32)
+        self.flags = gu.garbage_like(torch.empty((max(T, 1), R), dtype=torch.bool, device=gu.DEV)).view(torch.uint8)
+        self.off = torch.full((E + 1,), -3, **i32)
+        self.psum = torch.full((R,), -3, **i32)
+        self.channel_prefix = torch.full((R, channels), -3, **i32)
+        self.slot_rel = torch.full((max(T, 1), K), -3, **i32)
+        self.rank_slot_idx = torch.full((max(T, 1), K), -3, **i32)
+        # entries past the last token are never written: same fill on both sides
+        self.route_order = torch.full((max(lib.mi_ep_route_order_bytes(T, K) // 16, 1), 4), -3, **i32)
+
+    def tensors(self):
+        return [self.per_rank, self.per_expert, self.flags, self.off, self.psum, self.channel_prefix,
+                self.slot_rel, self.rank_slot_idx, self.route_order]
+
+
+def run_both(lib, topk_np, R, E, align, channels):
+    T, K = topk_np.shape
+    topk = torch.from_numpy(topk_np).to(gu.DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    want, got = LayoutOutputs(T, K, R, E, channels, lib), LayoutOutputs(T, K, R, E, channels, lib)
+    ws_bytes = lib.mi_ep_workspace_bytes(max(T, 1), K, E, R)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=gu.DEV)
+    _lib.check(lib.mi_ep_workspace_init(ws.data_ptr(), ws_bytes, stream), "workspace init")
+    _lib.check(lib.mi_ep_dispatch_layout(
+        topk.data_ptr(), T, K, R, E, align, channels, want.per_rank.data_ptr(), want.per_expert.data_ptr(),
+        want.flags.data_ptr(), want.off.data_ptr(), want.psum.data_ptr(), want.channel_prefix.data_ptr(),
+        want.slot_rel.data_ptr(), want.rank_slot_idx.data_ptr(), gu.RANK_SLOT_BASE, want.route_order.data_ptr(),
+        ws.data_ptr(), ws_bytes, stream), "mi_ep_dispatch_layout")
+    report = torch.zeros(1, dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.mi_ep_dispatch_layout_static(
+        topk.data_ptr(), T, K, R, E, align, channels, got.per_rank.data_ptr(), got.per_expert.data_ptr(),
+        got.flags.data_ptr(), got.off.data_ptr(), got.psum.data_ptr(), got.channel_prefix.data_ptr(),
+        got.slot_rel.data_ptr(), got.rank_slot_idx.data_ptr(), gu.RANK_SLOT_BASE, got.route_order.data_ptr(),
+        report.data_ptr(), stream), "mi_ep_dispatch_layout_static")
+    torch.cuda.synchronize()
+    _lib.check(lib.mi_ep_workspace_status(ws.data_ptr(), stream), "workspace status")
+    assert int(report.item()) == 0
+    for a, b in zip(want.tensors(), got.tensors()):
+        assert torch.equal(a, b)
+    return want
+
+
+def test_static_layout_matches_the_workspace_entry_point_on_calls_in_a_row(oracle):
+    lib = _lib.load()
+    # (T, K, R, E, alignment, channels): large first, then smaller inputs on the same scratch,
+    # with other column counts, so that status words of earlier calls lie under later ones.
+    shapes = [(8192, 8, 8, 256, 128, 16), (1000, 8, 8, 256, 1, 16), (4097, 4, 4, 64, 16, 8),
+              (300, 2, 2, 8, 1, 4), (8192, 8, 8, 256, 1, 16)]
+    for n, (T, K, R, E, align, channels) in enumerate(shapes):
+        print(f"call {n}: shape {(T, K, R, E)} alignment {align}", flush=True)
+        rng = np.random.default_rng(100 + n)
+        topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+        topk_np[rng.random((T, K)) < 0.05] = -1
+        want = run_both(lib, topk_np, R, E, align, channels)
+        # and the shared result is the checker's
+        per_rank, per_expert, flags = oracle.layout(topk_np, R, E)
+        off, _ = oracle.expert_offsets(per_expert, R, align)
+        np.testing.assert_array_equal(want.per_rank.cpu().numpy(), per_rank)
+        np.testing.assert_array_equal(want.per_expert.cpu().numpy(), per_expert)
+        np.testing.assert_array_equal(want.off.cpu().numpy(), off)
+        np.testing.assert_array_equal(want.flags.cpu().numpy()[:T], flags)
+
+
+def test_static_layout_refuses_shapes_beyond_its_scratch():
+    lib = _lib.load()
+    K, R, E = 2, 8, 1024
+    tiles = STATUS_WORDS // (E + R) + 1
+    T = tiles * 256
+    # nothing is launched, so no buffer is touched: null outputs are never reached
+    one = torch.zeros(8, dtype=torch.int64, device=gu.DEV)
+    rc = lib.mi_ep_dispatch_layout_static(one.data_ptr(), T, K, R, E, 1, 0, one.data_ptr(), one.data_ptr(),
+                                          one.data_ptr(), None, None, None, None, None, 0, None, None,
+                                          torch.cuda.current_stream().cuda_stream)
+    assert rc == E2BIG
+    assert "static scratch" in _lib.strerror(rc)
+    torch.cuda.synchronize()
+    assert int(one.sum().item()) == 0
