@@ -3,12 +3,14 @@
 
 One step = one pass of the three kernels over one batch of synthetic input that already sits
 in HBM: fused layout -> permute into the expert-contiguous buffer -> weighted combine of fresh
-bf16 expert outputs.  Prints one JSON line (see the keys below).  The CPU checker is timed on a
-bounded sample of the same workload as a reported baseline.
+bf16 expert outputs.  Inputs come from the same seeded generators the parity tests use
+(commbench_amd/workloads.py).  Prints one JSON line (see the keys below).  The CPU checker is
+timed on the same workload and inputs as a reported baseline.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config target|c2|c3|c4|c5]
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -19,6 +21,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBPS = 8000.0      # MI355X published HBM3E bandwidth
+KEEP_PAD_PAYLOAD = 1        # MI_EP_DISPATCH_KEEP_PAD_PAYLOAD
 
 
 def parse_args():
@@ -38,14 +41,36 @@ def parse_args():
                     help="skip the PCIe-inclusive pass through the host-pointer entry points")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short runs of the other configurations reported under other_configs")
+    ap.add_argument("--no-yardsticks", action="store_true",
+                    help="skip the linear copy / read / write streams measured beside the roofline")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
+
+
+_EXPERT_OUTPUTS = {}   # config name -> the longest generated y so far (shorter ones are prefixes of it)
+
+
+def fill_expert_outputs(cfg, y):
+    """Fills y ([rows, hidden] bf16 on the GPU) with wl.make_expert_outputs(cfg, rows), generated in
+    blocks of rows so that the float32 staging stays small (same generator, same stream).  Variants
+    of one configuration reuse what was generated before."""
+    from commbench_amd import workloads as wl
+    rows = y.shape[0]
+    have = _EXPERT_OUTPUTS.get(cfg.name)
+    if have is not None and have.shape[0] >= rows:
+        y.copy_(have[:rows])
+        return
+    rng = wl.rng_for(cfg, 2)
+    for i in range(0, rows, 8192):
+        n = min(8192, rows - i)
+        y[i:i + n].copy_(wl.bf16_normal(rng, n, cfg.hidden))
+    _EXPERT_OUTPUTS[cfg.name] = y.clone()
 
 
 class Workload:
     """Device buffers and raw C-ABI calls of one configuration (nothing allocates in a step)."""
 
-    def __init__(self, cfg, dev, rotate_x=1, expert_alignment=1):
+    def __init__(self, cfg, dev, rotate_x=1, expert_alignment=1, dispatch_flags=0):
         import torch
         from commbench_amd import _lib, workloads as wl
 
@@ -56,18 +81,14 @@ class Workload:
         self.num_routes = int((topk_np >= 0).sum())
         self.topk = torch.from_numpy(topk_np).to(dev)
         self.w = torch.from_numpy(w_np).to(dev)
-        gen = torch.Generator(device=dev).manual_seed(wl.SEED_BASE + cfg.config_id)
-        x = torch.randn((T, H), device=dev, generator=gen, dtype=torch.float32).to(torch.bfloat16)
-        self.scales = None
-        if cfg.payload == "fp8":
-            xf = x.to(torch.float32).view(T, H // 128, 128)
-            amax = xf.abs().amax(dim=2)
-            self.scales = torch.where(amax > 0, amax / 448.0, torch.ones_like(amax)).contiguous()
-            x = (xf / self.scales[:, :, None]).clamp_(-448, 448).to(torch.float8_e4m3fn).view(T, H)
-        self.x = x.contiguous()
+        x_cpu, scales_cpu = wl.make_payload(cfg)          # the tests' generator: seeded PCG64, N(0,1) as bf16
+        self.x_cpu, self.scales_cpu = x_cpu, scales_cpu
+        self.x = x_cpu.to(dev).contiguous()
+        self.scales = None if scales_cpu is None else scales_cpu.to(dev).contiguous()
         self.x_ring = [self.x] + [self.x.clone() for _ in range(max(0, rotate_x - 1))]
         self.step_index = 0
         self.align = expert_alignment
+        self.dispatch_flags = dispatch_flags
         cap = T * K + E * (expert_alignment - 1)
         self.cap = cap
         self.recv_x = torch.empty((cap, H), dtype=self.x.dtype, device=dev)
@@ -76,9 +97,7 @@ class Workload:
         # Expert outputs: a buffer of their own, so combine reads from HBM, not from lines the
         # permute just wrote.
         self.y = torch.empty((cap, H), dtype=torch.bfloat16, device=dev)
-        for i in range(0, cap, 8192):
-            n = min(8192, cap - i)
-            self.y[i:i + n] = torch.randn((n, H), device=dev, generator=gen).to(torch.bfloat16)
+        fill_expert_outputs(cfg, self.y)
         i32 = dict(dtype=torch.int32, device=dev)
         self.per_rank = torch.empty(R, **i32)
         self.per_expert = torch.empty(E, **i32)
@@ -98,6 +117,13 @@ class Workload:
         _lib.check(self.lib.mi_ep_workspace_init(self.ws.data_ptr(), ws_bytes, self.stream), "ws init")
         self.bytes = wl.algorithmic_bytes(T, H, E, K, R, self.num_routes,
                                           1 if cfg.payload == "fp8" else 2, cfg.num_scales)
+        # Bytes of the zero-filled pad rows (alignment > 1, payload not kept): extra writes on top of
+        # the algorithmic count.
+        counts = wl.np.bincount(topk_np[topk_np >= 0].ravel(), minlength=E)
+        pad_rows = int(((counts + expert_alignment - 1) // expert_alignment * expert_alignment - counts).sum())
+        zeroed = expert_alignment > 1 and not (dispatch_flags & KEEP_PAD_PAYLOAD)
+        self.pad_rows = pad_rows
+        self.padded_bytes = pad_rows * (cfg.row_bytes + cfg.num_scales * 4) if zeroed else 0
 
     def layout(self):
         c = self.cfg
@@ -105,7 +131,8 @@ class Workload:
             self.topk.data_ptr(), c.num_tokens, c.num_topk, c.num_ranks, c.num_experts, self.align, 0,
             self.per_rank.data_ptr(), self.per_expert.data_ptr(), self.in_rank.data_ptr(),
             self.off.data_ptr(), self.psum.data_ptr(), None, self.slot_rel.data_ptr(), None, 0,
-            self.route_order.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream), "layout")
+            self.route_order.data_ptr(), None, None, None, self.ws.data_ptr(), self.ws.numel(), self.stream),
+            "layout")
 
     def dispatch(self):
         c = self.cfg
@@ -118,13 +145,13 @@ class Workload:
             c.num_experts, self.align, c.row_bytes, c.num_scales, self.recv_x.data_ptr(),
             None if self.recv_scales is None else self.recv_scales.data_ptr(),
             self.src_map.data_ptr(), self.recv_idx.data_ptr(), self.recv_w.data_ptr(),
-            self.slot_map.data_ptr(), self.cap, 0, self.stream), "dispatch")
+            self.slot_map.data_ptr(), self.cap, self.dispatch_flags, self.stream), "dispatch")
 
     def combine(self):
         c = self.cfg
         self._lib.check(self.lib.mi_ep_combine(
-            self.y.data_ptr(), self.cap, self.slot_map.data_ptr(), self.w.data_ptr(), None, None, None,
-            c.num_tokens, c.num_topk, c.hidden, self.out.data_ptr(), None, self.stream), "combine")
+            self.y.data_ptr(), self.cap, self.slot_map.data_ptr(), self.w.data_ptr(), None, None, None, None,
+            c.num_tokens, c.num_topk, c.hidden, self.out.data_ptr(), None, None, self.stream), "combine")
 
     def step(self):
         self.layout()
@@ -132,21 +159,95 @@ class Workload:
         self.combine()
 
 
-def host_path(cfg, sample_tokens=2048):
-    """The same step through the host-pointer entry points (numpy in, numpy out) on a bounded
-    token sample: what a caller pays when the data lives in host memory.  Never `value`."""
+class RankWorkload:
+    """The same step in the reference's own receive format: one row per (token, destination rank),
+    K expert ids / gate weights and the source metadata per row; combine is the plain ordered sum of
+    a token's rows (mi_ep_dispatch_ranks, then mi_ep_combine over combine_map)."""
+
+    def __init__(self, cfg, dev):
+        import torch
+        from commbench_amd import _lib, workloads as wl
+
+        self.cfg, self.lib, self._lib = cfg, _lib.load(), _lib
+        T, K, E, R, H = cfg.num_tokens, cfg.num_topk, cfg.num_experts, cfg.num_ranks, cfg.hidden
+        topk_np, w_np = wl.make_routing(cfg)
+        valid = topk_np >= 0
+        ranks = wl.np.where(valid, topk_np // (E // R), -1)
+        self.num_rows = int(sum(len(set(r[r >= 0].tolist())) for r in ranks))   # distinct ranks per token
+        self.topk = torch.from_numpy(topk_np).to(dev)
+        self.w = torch.from_numpy(w_np).to(dev)
+        x_cpu, _ = wl.make_payload(cfg)
+        self.x = x_cpu.to(dev).contiguous()
+        cap = T * min(K, R)
+        self.cap = cap
+        i32 = dict(dtype=torch.int32, device=dev)
+        self.per_rank, self.per_expert = torch.empty(R, **i32), torch.empty(E, **i32)
+        self.in_rank = torch.empty((T, R), dtype=torch.bool, device=dev)
+        self.rank_slot_idx = torch.empty((T, K), **i32)
+        self.recv_x = torch.empty((cap, H), dtype=self.x.dtype, device=dev)
+        self.recv_idx = torch.empty((cap, K), dtype=torch.int64, device=dev)
+        self.recv_w = torch.empty((cap, K), dtype=torch.float32, device=dev)
+        self.meta = torch.empty((cap, 2 + K), **i32)
+        self.row_map, self.combine_map = torch.empty((T, K), **i32), torch.empty((T, K), **i32)
+        self.psum = torch.empty(R, **i32)
+        self.y = torch.empty((cap, H), dtype=torch.bfloat16, device=dev)
+        fill_expert_outputs(cfg, self.y)
+        self.out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+        ws_bytes = self.lib.mi_ep_workspace_bytes(T, K, E, R)
+        self.ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        self.stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(self.lib.mi_ep_workspace_init(self.ws.data_ptr(), ws_bytes, self.stream), "ws init")
+        n, row = self.num_rows, cfg.row_bytes
+        layout = T * K * 8 + T * R + (R + E) * 4 + T * K * 4
+        dispatch = T * row + n * row + T * K * 8 + T * K * 4 + T * K * 4 + n * (K * 8 + K * 4 + (2 + K) * 4) + 2 * T * K * 4
+        combine = n * H * 2 + T * H * 2 + T * K * 4
+        self.bytes = {"layout": layout, "dispatch": dispatch, "combine": combine, "total": layout + dispatch + combine}
+
+    def layout(self):
+        c = self.cfg
+        self._lib.check(self.lib.mi_ep_dispatch_layout(
+            self.topk.data_ptr(), c.num_tokens, c.num_topk, c.num_ranks, c.num_experts, 1, 0,
+            self.per_rank.data_ptr(), self.per_expert.data_ptr(), self.in_rank.data_ptr(), None, None, None, None,
+            self.rank_slot_idx.data_ptr(), 0, None, None, None, None, self.ws.data_ptr(), self.ws.numel(),
+            self.stream), "layout")
+
+    def dispatch(self):
+        c = self.cfg
+        self._lib.check(self.lib.mi_ep_dispatch_ranks(
+            self.x.data_ptr(), None, self.topk.data_ptr(), self.w.data_ptr(), self.rank_slot_idx.data_ptr(), 0,
+            self.per_rank.data_ptr(), None, c.num_tokens, c.num_topk, c.num_ranks, c.num_experts, c.row_bytes, 0,
+            0, 0, self.recv_x.data_ptr(), None, self.recv_idx.data_ptr(), self.recv_w.data_ptr(),
+            self.meta.data_ptr(), self.row_map.data_ptr(), self.combine_map.data_ptr(), self.psum.data_ptr(),
+            self.cap, self.stream), "dispatch_ranks")
+
+    def combine(self):
+        c = self.cfg
+        self._lib.check(self.lib.mi_ep_combine(
+            self.y.data_ptr(), self.cap, self.combine_map.data_ptr(), None, None, None, None, None,
+            c.num_tokens, c.num_topk, c.hidden, self.out.data_ptr(), None, None, self.stream), "combine")
+
+    def step(self):
+        self.layout()
+        self.dispatch()
+        self.combine()
+
+
+def host_path(cfg, wk, sample_tokens=2048):
+    """The same step through the host-pointer entry points (numpy in, numpy out) on the first
+    tokens of the same inputs: what a caller pays when the data lives in host memory.  Never `value`."""
     import numpy as np
-    from commbench_amd import ops, workloads as wl
-    topk_np, w_np = wl.make_routing(cfg)
+    import torch
+    from commbench_amd import ops
     n = min(sample_tokens, cfg.num_tokens)
-    topk_np, w_np = topk_np[:n], w_np[:n]
-    rng = np.random.default_rng(wl.SEED_BASE + cfg.config_id)
-    x = rng.integers(0, 1 << 16, size=(n, cfg.row_bytes // 2), dtype=np.uint16)
+    topk_np, w_np = wk.topk_np[:n], wk.w_np[:n]
+    x = wk.x_cpu[:n].contiguous().view(torch.uint8).numpy().reshape(n, -1)
+    scales = None if wk.scales_cpu is None else wk.scales_cpu[:n].contiguous().numpy()
     best = None
     for _ in range(3):
         t0 = time.perf_counter()
-        d = ops.host_dispatch(x, None, topk_np, w_np, cfg.num_experts, cfg.num_ranks)
-        y = d["recv_x"] if cfg.payload == "bf16" else np.zeros((d["recv_x"].shape[0], cfg.hidden), np.uint16)
+        d = ops.host_dispatch(x, scales, topk_np, w_np, cfg.num_experts, cfg.num_ranks)
+        y = (d["recv_x"].view(np.uint16) if cfg.payload == "bf16"
+             else np.zeros((d["recv_x"].shape[0], cfg.hidden), np.uint16))
         ops.host_combine(y, d["slot_map"], w_np)
         dt = time.perf_counter() - t0
         best = dt if best is None else min(best, dt)
@@ -156,28 +257,24 @@ def host_path(cfg, sample_tokens=2048):
                     "buffers allocated per call, best of 3"}
 
 
-def cpu_baseline(cfg, seconds):
-    """The CPU checker on a bounded token sample of the same workload, one thread and all the
-    host cores this job may use; returns the cpu_baseline object."""
+def cpu_baseline(cfg, wk, seconds):
+    """The CPU checker on the full workload with the benchmark's own inputs (same generators, same
+    seeds), one thread and all the host cores this job may use; returns the cpu_baseline object."""
     import numpy as np
-    from commbench_amd import workloads as wl
+    import torch
     from oracle import ep_oracle
 
-    sample_tokens = min(cfg.num_tokens, 1024)
-    topk_np, w_np = wl.make_routing(cfg)
-    topk_np, w_np = topk_np[:sample_tokens].copy(), w_np[:sample_tokens].copy()
-    rng = np.random.Generator(np.random.PCG64(1))
-    x = rng.integers(0, 1 << 16, size=(sample_tokens, cfg.row_bytes // 2), dtype=np.uint16)
-    scales = (rng.standard_normal((sample_tokens, cfg.num_scales)).astype(np.float32)
-              if cfg.num_scales else None)
-    rows = int((topk_np >= 0).sum())
-    y = ep_oracle.f32_to_bf16(rng.standard_normal((rows, cfg.hidden), dtype=np.float32))
+    T = cfg.num_tokens
+    topk_np, w_np = wk.topk_np, wk.w_np
+    x = wk.x_cpu.contiguous().view(torch.uint8).numpy().reshape(T, -1)
+    scales = None if wk.scales_cpu is None else wk.scales_cpu.numpy()
+    rows = wk.num_routes
+    y = wk.y[:rows].cpu().view(torch.int16).numpy().view(np.uint16)
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
     threads = max(1, min(threads, os.cpu_count() or 1, 16))
 
     def one_pass(nthreads):
-        res = ep_oracle.full_path(topk_np, w_np, x.view(np.uint8), scales, cfg.num_experts,
-                                  cfg.num_ranks, 1, nthreads)
+        res = ep_oracle.full_path(topk_np, w_np, x, scales, cfg.num_experts, cfg.num_ranks, 1, nthreads)
         ep_oracle.combine(y, res["slot_map"], w_np, num_threads=nthreads)
 
     def rate(nthreads, budget):
@@ -188,10 +285,10 @@ def cpu_baseline(cfg, seconds):
             n += 1
             dt = time.perf_counter() - t0
             if dt >= budget:
-                return n * sample_tokens / dt
+                return n * T / dt, n
 
-    single = rate(1, seconds * 0.5)
-    multi = rate(threads, seconds * 0.5) if threads > 1 else single
+    single, n1 = rate(1, seconds * 0.5)
+    multi, nm = rate(threads, seconds * 0.5) if threads > 1 else (single, n1)
     model = "unknown"
     try:
         with open("/proc/cpuinfo") as f:
@@ -204,9 +301,49 @@ def cpu_baseline(cfg, seconds):
     return {"value": multi, "unit": "tokens/s", "cores": threads, "kind": "port",
             "single_thread_value": single, "threads": threads, "host_nproc": os.cpu_count(),
             "host_cpu_model": model,
-            "sample": f"first {sample_tokens} tokens of the workload ({rows} routes): layout + "
-                      f"offsets + slot maps + permute + combine, repeated for ~{seconds:.0f} s "
-                      f"(half on 1 thread, half on {threads} OpenMP threads)"}
+            "sample": f"full workload, {T} tokens ({rows} routes), the benchmark's own inputs: layout + "
+                      f"offsets + slot maps + permute + combine; {n1} passes on 1 thread and {nm} passes on "
+                      f"{threads} OpenMP threads (~{seconds:.0f} s in all)"}
+
+
+def measured_traffic(kernel, workload_name):
+    """HBM bytes per launch of `kernel` from the committed counter runs, or None when the kernel
+    sources have changed since they were taken (the file records their hashes)."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        rec = json.load(f)
+    for name, want in rec.get("source_sha16", {}).items():
+        src = os.path.join(ROOT, "commbench_amd", "csrc", name)
+        if not os.path.exists(src) or hashlib.sha256(open(src, "rb").read()).hexdigest()[:16] != want:
+            return None
+    return rec.get(workload_name, {}).get(kernel)
+
+
+def time_steps(torch, wk, warmup, steps):
+    for _ in range(warmup):
+        wk.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        wk.step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def kernel_medians(torch, wk, reps):
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(reps)]
+    for ev in marks:
+        ev[0].record()
+        wk.layout()
+        ev[1].record()
+        wk.dispatch()
+        ev[2].record()
+        wk.combine()
+        ev[3].record()
+    torch.cuda.synchronize()
+    return marks
 
 
 def main():
@@ -218,7 +355,7 @@ def main():
         sys.exit(2)
 
     import torch
-    from commbench_amd import workloads as wl
+    from commbench_amd import ops, workloads as wl
 
     cfg = wl.CONFIGS[args.config]
     dev = "cuda:0"
@@ -226,18 +363,11 @@ def main():
     wk = Workload(cfg, dev, args.rotate_x)
     T = cfg.num_tokens
 
-    for _ in range(args.warmup):
+    # Load before any measurement: the device idled while the inputs were generated on the CPU, and its
+    # clocks take about 20 ms of work to settle.
+    for _ in range(80):
         wk.step()
     torch.cuda.synchronize()
-
-    # Timed region: exactly `steps` steps, back to back on one stream.
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        wk.step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
 
     # The same steps with the source rows cycling through three buffers, so that they come from
     # HBM instead of the 256 MB memory-side cache that keeps a single re-read source resident.
@@ -282,24 +412,17 @@ def main():
 
     # Per-kernel durations: the same steps again with HIP events on the launch stream
     # bracketing every kernel (kept out of the region above, where they would add gaps).
-    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
     torch.cuda.synchronize()
-    for ev in marks:
-        ev[0].record()
-        wk.layout()
-        ev[1].record()
-        wk.dispatch()
-        ev[2].record()
-        wk.combine()
-        ev[3].record()
-    torch.cuda.synchronize()
+    marks = kernel_medians(torch, wk, args.steps)
 
     # Kernel symbols as rocprofv3 reports them; the combine schedule depends on the shape
     # (persistent LDS-staged kernel from 16 tokens per compute unit and 2 KiB rows upwards).
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    traits = ops.device_traits()
+    cus = traits["compute_units"]
     staged = T >= 16 * cus and 2048 <= cfg.hidden * 2 <= 160 * 1024
-    by_destination = wk.lib.mi_ep_dispatch_schedule_for(T, cfg.num_topk, cfg.num_experts, cfg.row_bytes) == 2
-    names = ["ep_layout_fused_kernel", "ep_permute_tiles_kernel" if by_destination else "ep_permute_kernel",
+    schedule = ops.dispatch_schedule_for(T, cfg.num_topk, cfg.num_experts, cfg.row_bytes)
+    names = ["ep_layout_fused_kernel",
+             "ep_permute_tiles_kernel" if schedule == "destination" else "ep_permute_kernel",
              "ep_combine_staged_kernel" if staged else "ep_combine_kernel"]
     per_step = {n: sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for ev in marks) for i, n in enumerate(names)}
     kernel_us = {n: sum(v) / len(v) for n, v in per_step.items()}
@@ -311,36 +434,47 @@ def main():
 
     # Measured ceilings next to the nominal peak: 16-byte streaming copy, read-only and
     # write-only passes over the same 0.94-1 GiB buffers.
-    lib, check = wk.lib, wk._lib.check
-    src = wk.y.view(torch.uint8).reshape(-1)[: 1 << 30]
-    dst = wk.recv_x.view(torch.uint8).reshape(-1)[: src.numel()]
-    src = src[: dst.numel()]
-    nbytes = src.numel() - src.numel() % 16
-    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    copy_gbps = read_gbps = write_gbps = None
+    if not args.no_yardsticks:
+        lib, check = wk.lib, wk._lib.check
+        src = wk.y.view(torch.uint8).reshape(-1)[: 1 << 30]
+        dst = wk.recv_x.view(torch.uint8).reshape(-1)[: src.numel()]
+        src = src[: dst.numel()]
+        nbytes = src.numel() - src.numel() % 16
+        sink = torch.zeros(1, dtype=torch.int32, device=dev)
 
-    def timed(fn, moved_bytes, iters=10):
-        for _ in range(3):
-            fn()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return moved_bytes * iters / (e0.elapsed_time(e1) * 1e-3) / 1e9
+        def timed(fn, moved_bytes, iters=10):
+            for _ in range(3):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return moved_bytes * iters / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
-    copy_gbps = timed(lambda: check(lib.mi_ep_copy_yardstick(dst.data_ptr(), src.data_ptr(), nbytes, wk.stream),
-                                    "copy yardstick"), 2 * nbytes)
-    read_gbps = timed(lambda: check(lib.mi_ep_read_yardstick(src.data_ptr(), nbytes, sink.data_ptr(), wk.stream),
-                                    "read yardstick"), nbytes)
-    write_gbps = timed(lambda: check(lib.mi_ep_write_yardstick(dst.data_ptr(), nbytes, wk.stream),
-                                     "write yardstick"), nbytes)
+        copy_gbps = timed(lambda: check(lib.mi_ep_copy_yardstick(dst.data_ptr(), src.data_ptr(), nbytes, wk.stream),
+                                        "copy yardstick"), 2 * nbytes)
+        read_gbps = timed(lambda: check(lib.mi_ep_read_yardstick(src.data_ptr(), nbytes, sink.data_ptr(), wk.stream),
+                                        "read yardstick"), nbytes)
+        write_gbps = timed(lambda: check(lib.mi_ep_write_yardstick(dst.data_ptr(), nbytes, wk.stream),
+                                         "write yardstick"), nbytes)
 
-    traffic = None
-    traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(traffic_file):
-        with open(traffic_file) as f:
-            traffic = json.load(f).get(cfg.name, {}).get(dominant)
+    # The headline region comes last of the GPU measurements: after an idle period (the CPU-side
+    # input generation above) the device's power management needs about 20 ms of load to reach its
+    # sustained clocks (measured here: 389 -> 365 -> 356 us per step over the first 15 ms), and the
+    # passes above provide that load.  W warm-up steps, a synchronisation, exactly K timed steps back
+    # to back on one stream, a synchronisation.
+    for _ in range(args.warmup):
+        wk.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        wk.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
 
     result = {
         "metric": "dispatch+combine tokens/s and achieved HBM GB/s (% of peak), 1 MI355X",
@@ -363,6 +497,8 @@ def main():
             "num_tokens": T, "hidden": cfg.hidden, "num_experts": cfg.num_experts,
             "num_topk": cfg.num_topk, "num_ranks": cfg.num_ranks, "payload": cfg.payload,
             "source_buffers": args.rotate_x,
+            "inputs": "commbench_amd.workloads generators (PCG64 seeded 0xC0FFEE + config id): "
+                      "make_routing, make_payload, make_expert_outputs",
         },
         "hbm_gbps_whole_step": wk.bytes["total"] / (ms_per_step * 1e-3) / 1e9,
         "hbm_frac_whole_step": wk.bytes["total"] / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
@@ -373,6 +509,7 @@ def main():
             "hbm_frac_whole_step": wk.bytes["total"] / (cold_ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
             "note": "source rows cycled through 3 buffers so that they are read from HBM"},
         "algorithmic_bytes": wk.bytes,
+        "device_traits": traits,
         "kernel_us": kernel_us,
         "kernel_us_stats": kernel_us_stats,
         "kernel_gbps": {n: kernel_bytes[n] / (kernel_us[n] * 1e-6) / 1e9 for n in names},
@@ -381,54 +518,55 @@ def main():
         "write_yardstick_gbps": write_gbps,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBPS,
-                     "traffic": traffic},
+                     "traffic": measured_traffic(dominant, cfg.name)},
     }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg, wk, args.cpu_seconds)
+    if not args.no_host_path:
+        result["host_path"] = host_path(cfg, wk)
     if not args.no_other_configs:
         # Short runs of the other configurations, same step, for reference beside the headline.
         del wk
         torch.cuda.empty_cache()
         others = {}
         # "<name>@128": the same shape with expert segments padded to 128 rows, as the reference's
-        # harness asks of dispatch (example080 build_and_run.py:718); the zero-filled pad rows are
-        # extra bytes on top of the algorithmic count, so its fraction understates the traffic.
-        for name in ("c2", "c3", "c4", "c5", "target", cfg.name + "@128"):
+        # harness asks of dispatch (example080 build_and_run.py:718).  With zero-filled pads the fill
+        # is extra traffic (padded_bytes) on top of the algorithmic count; "@128/keep" leaves the pad
+        # payload alone, which is what the reference's receive buffer does.
+        # "<name>/ranks": the reference's per-rank receive format.
+        variants = [("c2", 1, 0), ("c3", 1, 0), ("c4", 1, 0), ("c5", 1, 0), ("target", 1, 0),
+                    (cfg.name + "@128", 128, 0), (cfg.name + "@128/keep", 128, KEEP_PAD_PAYLOAD),
+                    (cfg.name + "/ranks", 1, 0)]
+        for name, align, flags in variants:
             if name == cfg.name:
                 continue
-            ocfg = wl.CONFIGS[name.split("@")[0]]
-            owk = Workload(ocfg, dev, expert_alignment=128 if name.endswith("@128") else 1)
-            for _ in range(10):
-                owk.step()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(100):
-                owk.step()
-            torch.cuda.synchronize()
-            us = (time.perf_counter() - t0) * 1e6 / 100
-            omarks = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(30)]
-            for ev in omarks:
-                ev[0].record()
-                owk.layout()
-                ev[1].record()
-                owk.dispatch()
-                ev[2].record()
-                owk.combine()
-                ev[3].record()
-            torch.cuda.synchronize()
+            ocfg = wl.CONFIGS[name.split("@")[0].split("/")[0]]
+            ranks_format = name.endswith("/ranks")
+            owk = RankWorkload(ocfg, dev) if ranks_format else Workload(ocfg, dev, expert_alignment=align,
+                                                                         dispatch_flags=flags)
+            us = time_steps(torch, owk, 60, 100) * 1e6      # 60 steps: past the clock ramp that follows idle
+            omarks = kernel_medians(torch, owk, 30)
             median = lambda i: sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for ev in omarks)[len(omarks) // 2]
-            others[name] = {"us_per_step": us, "tokens_per_s": ocfg.num_tokens / (us * 1e-6),
-                            "kernel_us_median": {"layout": median(0), "dispatch": median(1), "combine": median(2)},
-                            "dispatch_schedule": owk.lib.mi_ep_dispatch_schedule_for(
-                                ocfg.num_tokens, ocfg.num_topk, ocfg.num_experts, ocfg.row_bytes),
-                            "hbm_gbps_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9,
-                            "hbm_frac_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS,
-                            "num_routes": owk.num_routes}
+            entry = {"us_per_step": us, "tokens_per_s": ocfg.num_tokens / (us * 1e-6),
+                     "kernel_us_median": {"layout": median(0), "dispatch": median(1), "combine": median(2)},
+                     "algorithmic_bytes": owk.bytes["total"],
+                     "hbm_gbps_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9,
+                     "hbm_frac_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS}
+            if ranks_format:
+                entry["num_rows"] = owk.num_rows
+            else:
+                entry["num_routes"] = owk.num_routes
+                entry["dispatch_schedule"] = ops.dispatch_schedule_for(ocfg.num_tokens, ocfg.num_topk,
+                                                                       ocfg.num_experts, ocfg.row_bytes)
+                if align > 1:
+                    entry["pad_rows"] = owk.pad_rows
+                    entry["padded_bytes"] = owk.padded_bytes
+                    entry["hbm_frac_with_pads"] = ((owk.bytes["total"] + owk.padded_bytes) / (us * 1e-6) / 1e9
+                                                   / PEAK_HBM_GBPS)
+            others[name] = entry
             del owk
             torch.cuda.empty_cache()
         result["other_configs"] = others
-    if not args.no_host_path:
-        result["host_path"] = host_path(cfg)
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
     print(json.dumps(result))
 
 

@@ -18,13 +18,15 @@ SIGNATURES = {
     "mi_ep_workspace_bytes": (_size, [_int, _int, _int, _int]),
     "mi_ep_workspace_init": (_int, [_vp, _size, _vp]),
     "mi_ep_workspace_status": (_int, [_vp, _vp]),
-    "mi_ep_set_wait_limit": (_int, [ctypes.c_uint]),
-    "mi_ep_set_dispatch_schedule": (_int, [_int]),
-    "mi_ep_dispatch_schedule_for": (_int, [_int, _int, _int, _int]),
+    "mi_ep_workspace_set_wait_limit": (_int, [_vp, ctypes.c_uint, _vp]),
+    "mi_ep_device_traits": (_int, [_c_int_p, _c_int_p, _c_int_p, _vp]),
+    "mi_ep_dispatch_schedule_for": (_int, [_int, _int, _int, _int, _int, _int]),
     "mi_ep_dispatch_layout": (_int, [_vp, _int, _int, _int, _int, _int, _int,
-                                     _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _size, _vp]),
+                                     _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp,
+                                     _vp, _size, _vp]),
     "mi_ep_dispatch_layout_static": (_int, [_vp, _int, _int, _int, _int, _int, _int,
-                                            _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp]),
+                                            _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp,
+                                            _vp, _vp]),
     "mi_ep_route_order_bytes": (_size, [_int, _int]),
     "mi_ep_dispatch": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int,
                               _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
@@ -34,11 +36,17 @@ SIGNATURES = {
                                              _vp]),
     "mi_ep_dispatch_ranks": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _int, _int, _int, _int, _int,
                                     _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
-    "mi_ep_combine_rank_weights": (_int, [_vp, _vp, _int, _int, _int, _vp, _vp]),
+    "mi_ep_dispatch_ranks_strided_scales": (_int, [_vp, _vp, ctypes.c_longlong, ctypes.c_longlong, _vp, _vp, _vp,
+                                                   _int, _vp, _vp, _int, _int, _int, _int, _int, _int, _int, _int,
+                                                   _vp, _vp, ctypes.c_longlong, ctypes.c_longlong, _vp, _vp, _vp,
+                                                   _vp, _vp, _vp, _int, _vp]),
+    "mi_ep_combine_rank_weights": (_int, [_vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp]),
     "mi_ep_dispatch_cached": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _int, _vp]),
     "mi_ep_pull_indices": (_int, [_vp, _int, _int, _vp, _vp]),
-    "mi_ep_combine": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp]),
+    "mi_ep_combine": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp, _vp]),
     "mi_ep_host_get_dispatch_layout": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int]),
+    "mi_ep_host_dispatch_layout": (_int, [_vp, _int, _int, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp,
+                                          _vp, _vp, _int, _vp, _vp, _vp, _vp]),
     "mi_ep_host_dispatch": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _int,
                                    _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int]),
     "mi_ep_host_combine": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]),

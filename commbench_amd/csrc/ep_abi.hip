@@ -1,7 +1,8 @@
 // extern "C" boundary of the gfx950 dispatch core: argument checks on the host,
 // then kernel launches.  No allocation, no synchronisation (except
-// mi_ep_workspace_status, which says so), no process-wide state apart from the
-// wait limit of the test hook.
+// mi_ep_workspace_status, which says so) and no mutable process-wide state: what
+// varies per caller travels in arguments or in the caller's workspace; the only
+// file-scope data are per-device caches of hardware facts that never change.
 #include "../../include/mi_ep.h"
 
 #include <atomic>
@@ -32,83 +33,12 @@ inline int num_tiles_for(int num_tokens) { return (num_tokens + kTileTokens - 1)
 
 inline int status_of(hipError_t e) { return e == hipSuccess ? MI_EP_OK : static_cast<int>(e); }
 
-// Bounded device-side wait: polls spaced by s_sleep, roughly a microsecond apart,
-// so a few seconds before a launch gives up and flags the workspace.
-constexpr uint32_t kSpinLimit = 1u << 22;
-std::atomic<uint32_t> g_spin_limit{kSpinLimit};  // only ever changed by the test hook
-std::atomic<int> g_permute_schedule{kPermuteAuto};
-
-// Argument checks and launch shared by mi_ep_dispatch_layout (caller's workspace) and
-// mi_ep_dispatch_layout_static (the library's static scratch); `workspace_words` is the number of
-// status words behind the workspace header.
-int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
-                       int num_experts, int expert_alignment, int num_channels,
-                       int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
-                       int* expert_offsets, int* psum_rank_rows, int* channel_prefix_matrix,
-                       int* slot_rel, int* rank_slot_idx, int rank_slot_base, int* route_order,
-                       void* workspace, size_t workspace_bytes, int too_small_code,
-                       int* timeout_report, void* stream) {
-  if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
-  if (expert_alignment < 1) return MI_EP_EINVAL;
-  if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
-  if (channel_prefix_matrix != nullptr && (num_channels < 1 || num_channels > 4096)) return MI_EP_EINVAL;
-  if (psum_rank_rows != nullptr && expert_offsets == nullptr) return MI_EP_EINVAL;
-  // Padded totals must stay inside int32.
-  if ((static_cast<long long>(num_tokens) * num_topk +
-       static_cast<long long>(num_experts) * (expert_alignment - 1)) >= (1LL << 31))
-    return MI_EP_EINVAL;
-  hipStream_t s = as_stream(stream);
-
-  if (num_tokens == 0) {
-    // Nothing to scan: every output is zero.
-    hipError_t e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_rank), num_ranks, 0u, s);
-    if (e == hipSuccess)
-      e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_expert), num_experts, 0u, s);
-    if (e == hipSuccess && expert_offsets != nullptr)
-      e = launch_fill_u32(reinterpret_cast<uint32_t*>(expert_offsets), num_experts + 1, 0u, s);
-    if (e == hipSuccess && psum_rank_rows != nullptr)
-      e = launch_fill_u32(reinterpret_cast<uint32_t*>(psum_rank_rows), num_ranks, 0u, s);
-    if (e == hipSuccess && channel_prefix_matrix != nullptr)
-      e = launch_fill_u32(reinterpret_cast<uint32_t*>(channel_prefix_matrix),
-                          static_cast<size_t>(num_ranks) * num_channels, 0u, s);
-    return status_of(e);
-  }
-
-  if (topk_idx == nullptr || is_token_in_rank == nullptr || workspace == nullptr) return MI_EP_EINVAL;
-  if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
-  if (!aligned16(route_order)) return MI_EP_EINVAL;
-  if (workspace_bytes < mi_ep_workspace_bytes(num_tokens, num_topk, num_experts, num_ranks))
-    return too_small_code;
-
-  LayoutArgs a{};
-  a.topk_idx = topk_idx;
-  a.num_tokens_per_rank = num_tokens_per_rank;
-  a.num_tokens_per_expert = num_tokens_per_expert;
-  a.is_token_in_rank = reinterpret_cast<uint8_t*>(is_token_in_rank);
-  a.expert_offsets = expert_offsets;
-  a.psum_rank_rows = psum_rank_rows;
-  a.channel_prefix_matrix = channel_prefix_matrix;
-  a.slot_rel = slot_rel;
-  a.rank_slot_idx = rank_slot_idx;
-  a.rank_slot_base = rank_slot_base;
-  a.route_order = route_order;
-  a.ws = static_cast<LayoutWorkspace*>(workspace);
-  a.timeout_report = timeout_report;
-  a.num_tokens = num_tokens;
-  a.num_topk = num_topk;
-  a.num_ranks = num_ranks;
-  a.num_experts = num_experts;
-  a.experts_per_rank = num_experts / num_ranks;
-  a.expert_alignment = expert_alignment;
-  a.num_channels = num_channels;
-  a.num_tiles = num_tiles_for(num_tokens);
-  a.expert_bits = 1;
-  while ((1 << a.expert_bits) < num_experts) ++a.expert_bits;
-  a.inv_topk = ((1u << 19) + num_topk - 1) / num_topk;
-  a.inv_experts_per_rank = ((1u << 22) + a.experts_per_rank - 1) / a.experts_per_rank;
-  a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
-  return status_of(launch_layout_fused(a, s));
+inline bool route_count_ok(int num_tokens, int num_topk) {
+  return num_tokens >= 0 && num_topk > 0 && num_topk <= MI_EP_MAX_TOPK &&
+         static_cast<long long>(num_tokens) * num_topk < (1LL << 30);
 }
+
+constexpr int kScheduleFlags = MI_EP_DISPATCH_BY_TOKEN | MI_EP_DISPATCH_BY_DESTINATION;
 
 // ---- scratch of the allocation-free layout entry point ------------------------------------
 // One copy per GPU, held until the process ends: the layout workspace (256-byte header + status
@@ -137,6 +67,91 @@ int static_scratch_of_current_device(void** out) {
   }
   *out = p;
   return MI_EP_OK;
+}
+
+// Argument checks and launch shared by mi_ep_dispatch_layout (caller's workspace) and
+// mi_ep_dispatch_layout_static (workspace == nullptr and use_static_scratch: the library's static
+// scratch of the current device, resolved after the argument checks).
+int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
+                       int num_experts, int expert_alignment, int num_channels,
+                       int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
+                       int* expert_offsets, int* psum_rank_rows, int* channel_prefix_matrix,
+                       int* slot_rel, int* rank_slot_idx, int rank_slot_base, int* route_order,
+                       int* tile_rank_counts, int64_t* copied_topk_idx, int* cumulative_expert_stats,
+                       void* workspace, size_t workspace_bytes, bool use_static_scratch,
+                       int* timeout_report, void* stream) {
+  if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
+  // Shapes beyond the static array are refused before anything else is looked at.
+  if (use_static_scratch &&
+      static_cast<size_t>(num_tiles_for(num_tokens)) * static_cast<size_t>(num_experts + num_ranks) > kStaticStatusWords)
+    return MI_EP_E2BIG;
+  if (expert_alignment < 1) return MI_EP_EINVAL;
+  if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
+  if (channel_prefix_matrix != nullptr && (num_channels < 1 || num_channels > 4096)) return MI_EP_EINVAL;
+  if (psum_rank_rows != nullptr && expert_offsets == nullptr) return MI_EP_EINVAL;
+  // Padded totals must stay inside int32.
+  if ((static_cast<long long>(num_tokens) * num_topk +
+       static_cast<long long>(num_experts) * (expert_alignment - 1)) >= (1LL << 31))
+    return MI_EP_EINVAL;
+  if (num_tokens > 0 && (topk_idx == nullptr || is_token_in_rank == nullptr)) return MI_EP_EINVAL;
+  if (!aligned16(route_order)) return MI_EP_EINVAL;
+  hipStream_t s = as_stream(stream);
+  if (use_static_scratch && num_tokens > 0) {
+    const int rc = static_scratch_of_current_device(&workspace);
+    if (rc != MI_EP_OK) return rc;
+    workspace_bytes = kStaticScratchBytes;
+  }
+
+  if (num_tokens == 0) {
+    // Nothing to scan: every output is zero.
+    hipError_t e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_rank), num_ranks, 0u, s);
+    if (e == hipSuccess)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(num_tokens_per_expert), num_experts, 0u, s);
+    if (e == hipSuccess && expert_offsets != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(expert_offsets), num_experts + 1, 0u, s);
+    if (e == hipSuccess && psum_rank_rows != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(psum_rank_rows), num_ranks, 0u, s);
+    if (e == hipSuccess && channel_prefix_matrix != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(channel_prefix_matrix),
+                          static_cast<size_t>(num_ranks) * num_channels, 0u, s);
+    return status_of(e);
+  }
+
+  if (workspace == nullptr) return MI_EP_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
+  if (workspace_bytes < mi_ep_workspace_bytes(num_tokens, num_topk, num_experts, num_ranks))
+    return MI_EP_ENOSPC;
+
+  LayoutArgs a{};
+  a.topk_idx = topk_idx;
+  a.num_tokens_per_rank = num_tokens_per_rank;
+  a.num_tokens_per_expert = num_tokens_per_expert;
+  a.is_token_in_rank = reinterpret_cast<uint8_t*>(is_token_in_rank);
+  a.expert_offsets = expert_offsets;
+  a.psum_rank_rows = psum_rank_rows;
+  a.channel_prefix_matrix = channel_prefix_matrix;
+  a.slot_rel = slot_rel;
+  a.rank_slot_idx = rank_slot_idx;
+  a.rank_slot_base = rank_slot_base;
+  a.route_order = route_order;
+  a.tile_rank_counts = tile_rank_counts;
+  a.copied_topk_idx = copied_topk_idx;
+  a.cumulative_expert_stats = cumulative_expert_stats;
+  a.ws = static_cast<LayoutWorkspace*>(workspace);
+  a.timeout_report = timeout_report;
+  a.num_tokens = num_tokens;
+  a.num_topk = num_topk;
+  a.num_ranks = num_ranks;
+  a.num_experts = num_experts;
+  a.experts_per_rank = num_experts / num_ranks;
+  a.expert_alignment = expert_alignment;
+  a.num_channels = num_channels;
+  a.num_tiles = num_tiles_for(num_tokens);
+  a.expert_bits = 1;
+  while ((1 << a.expert_bits) < num_experts) ++a.expert_bits;
+  a.inv_topk = ((1u << 19) + num_topk - 1) / num_topk;
+  a.inv_experts_per_rank = ((1u << 22) + a.experts_per_rank - 1) / a.experts_per_rank;
+  return status_of(launch_layout_fused(a, s));
 }
 
 }  // namespace
@@ -184,6 +199,12 @@ int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream) 
                                    as_stream(stream)));
 }
 
+int mi_ep_workspace_set_wait_limit(void* workspace, unsigned int max_polls, void* stream) {
+  if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
+  LayoutWorkspace* ws = static_cast<LayoutWorkspace*>(workspace);
+  return status_of(launch_fill_u32(&ws->wait_limit, 1, max_polls, as_stream(stream)));
+}
+
 int mi_ep_workspace_status(const void* workspace, void* stream) {
   if (workspace == nullptr) return MI_EP_EINVAL;
   LayoutWorkspace header;
@@ -195,14 +216,18 @@ int mi_ep_workspace_status(const void* workspace, void* stream) {
   return header.timed_out != 0 ? MI_EP_ETIMEDOUT : MI_EP_OK;
 }
 
-int mi_ep_set_dispatch_schedule(int schedule) {
-  if (schedule != kPermuteAuto && schedule != kPermuteByToken && schedule != kPermuteByDestination)
-    return MI_EP_EINVAL;
-  g_permute_schedule.store(schedule, std::memory_order_relaxed);
+int mi_ep_device_traits(int* compute_units, int* dies, int* l2_bytes, void* stream) {
+  DeviceTraits t{};
+  const hipError_t e = device_traits(as_stream(stream), &t);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (compute_units != nullptr) *compute_units = t.compute_units;
+  if (dies != nullptr) *dies = t.dies;
+  if (l2_bytes != nullptr) *l2_bytes = t.l2_bytes;
   return MI_EP_OK;
 }
 
-int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, int row_bytes) {
+int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, int row_bytes, int dies,
+                                int l2_bytes) {
   if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK || num_experts <= 0 ||
       num_experts > MI_EP_MAX_EXPERTS || row_bytes <= 0 || row_bytes % 16 != 0)
     return MI_EP_EINVAL;
@@ -211,7 +236,10 @@ int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, i
   a.num_topk = num_topk;
   a.num_experts = num_experts;
   a.row_vecs = row_bytes / 16;
-  return destination_order_pays(a) ? kPermuteByDestination : kPermuteByToken;
+  DeviceTraits t{};
+  t.dies = dies;
+  t.l2_bytes = l2_bytes;
+  return destination_order_pays(a, t) ? MI_EP_DISPATCH_BY_DESTINATION : MI_EP_DISPATCH_BY_TOKEN;
 }
 
 size_t mi_ep_route_order_bytes(int num_tokens, int num_topk) {
@@ -219,23 +247,19 @@ size_t mi_ep_route_order_bytes(int num_tokens, int num_topk) {
   return static_cast<size_t>(num_tiles_for(num_tokens)) * kTileTokens * num_topk * 4 * sizeof(int);
 }
 
-int mi_ep_set_wait_limit(unsigned int max_polls) {
-  g_spin_limit.store(max_polls == 0 ? kSpinLimit : max_polls, std::memory_order_relaxed);
-  return MI_EP_OK;
-}
-
 int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
                           int num_experts, int expert_alignment, int num_channels,
                           int* num_tokens_per_rank, int* num_tokens_per_expert,
                           bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
                           int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
-                          int rank_slot_base, int* route_order, void* workspace,
+                          int rank_slot_base, int* route_order, int* tile_rank_counts,
+                          int64_t* copied_topk_idx, int* cumulative_expert_stats, void* workspace,
                           size_t workspace_bytes, void* stream) {
   return dispatch_layout_on(topk_idx, num_tokens, num_topk, num_ranks, num_experts, expert_alignment,
                             num_channels, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank,
                             expert_offsets, psum_rank_rows, channel_prefix_matrix, slot_rel, rank_slot_idx,
-                            rank_slot_base, route_order, workspace, workspace_bytes, MI_EP_ENOSPC, nullptr,
-                            stream);
+                            rank_slot_base, route_order, tile_rank_counts, copied_topk_idx,
+                            cumulative_expert_stats, workspace, workspace_bytes, false, nullptr, stream);
 }
 
 int mi_ep_dispatch_layout_static(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
@@ -243,35 +267,29 @@ int mi_ep_dispatch_layout_static(const int64_t* topk_idx, int num_tokens, int nu
                                  int* num_tokens_per_rank, int* num_tokens_per_expert,
                                  bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
                                  int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
-                                 int rank_slot_base, int* route_order, int* timeout_report, void* stream) {
-  // The shape check comes first so that an oversized request is refused before anything else.
-  if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
-  if (static_cast<size_t>(num_tiles_for(num_tokens)) * static_cast<size_t>(num_experts + num_ranks) >
-      kStaticStatusWords)
-    return MI_EP_E2BIG;
-  void* ws = nullptr;
-  const int rc = static_scratch_of_current_device(&ws);
-  if (rc != MI_EP_OK) return rc;
+                                 int rank_slot_base, int* route_order, int* tile_rank_counts,
+                                 int64_t* copied_topk_idx, int* cumulative_expert_stats,
+                                 int* timeout_report, void* stream) {
   // Nothing needs clearing between calls: the scratch starts zeroed when the code object is
   // loaded (an initialised workspace), and every launch leaves the ticket word ready for the
   // next and tags its status words with a fresh generation.
   return dispatch_layout_on(topk_idx, num_tokens, num_topk, num_ranks, num_experts, expert_alignment,
                             num_channels, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank,
                             expert_offsets, psum_rank_rows, channel_prefix_matrix, slot_rel, rank_slot_idx,
-                            rank_slot_base, route_order, ws, kStaticScratchBytes, MI_EP_E2BIG,
-                            timeout_report, stream);
+                            rank_slot_base, route_order, tile_rank_counts, copied_topk_idx,
+                            cumulative_expert_stats, nullptr, 0, true, timeout_report, stream);
 }
 
 int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long long x_scales_token_stride,
                                   long long x_scales_hidden_stride, const int64_t* topk_idx,
-                   const float* topk_weights, const int* expert_offsets, const int* slot_rel,
-                   const int* route_order, const int* num_tokens_per_expert, int num_tokens, int num_topk,
-                   int num_experts, int expert_alignment, int row_bytes, int num_scales,
-                   void* recv_x, float* recv_scales, long long recv_scales_token_stride,
-                   long long recv_scales_hidden_stride, int* recv_src_map, int64_t* recv_topk_idx,
-                   float* recv_topk_weights, int* slot_map, int capacity_rows, int flags,
-                   void* stream) {
-  if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK) return MI_EP_EINVAL;
+                                  const float* topk_weights, const int* expert_offsets, const int* slot_rel,
+                                  const int* route_order, const int* num_tokens_per_expert, int num_tokens,
+                                  int num_topk, int num_experts, int expert_alignment, int row_bytes,
+                                  int num_scales, void* recv_x, float* recv_scales,
+                                  long long recv_scales_token_stride, long long recv_scales_hidden_stride,
+                                  int* recv_src_map, int64_t* recv_topk_idx, float* recv_topk_weights,
+                                  int* slot_map, int capacity_rows, int flags, void* stream) {
+  if (!route_count_ok(num_tokens, num_topk)) return MI_EP_EINVAL;
   if (num_experts <= 0 || num_experts > MI_EP_MAX_EXPERTS || expert_alignment < 1) return MI_EP_EINVAL;
   if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
   if (expert_offsets == nullptr || recv_src_map == nullptr) return MI_EP_EINVAL;
@@ -283,10 +301,15 @@ int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long lon
   if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
   if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
   if (expert_alignment > 1 && num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
-  if ((flags & ~MI_EP_DISPATCH_KEEP_PAD_PAYLOAD) != 0) return MI_EP_EINVAL;
+  if ((flags & ~(MI_EP_DISPATCH_KEEP_PAD_PAYLOAD | kScheduleFlags)) != 0) return MI_EP_EINVAL;
+  if ((flags & kScheduleFlags) == kScheduleFlags) return MI_EP_EINVAL;  // one copy kernel at most
+  if ((flags & MI_EP_DISPATCH_BY_DESTINATION) != 0 && route_order == nullptr && num_tokens > 0)
+    return MI_EP_EINVAL;
   if (num_scales > 0 && (x_scales_token_stride < 0 || x_scales_hidden_stride < 0 ||
                          recv_scales_token_stride < 0 || recv_scales_hidden_stride < 0))
     return MI_EP_EINVAL;
+  // Pad rows are addressed as expert * (alignment - 1) + index in int.
+  if (static_cast<long long>(num_experts) * (expert_alignment - 1) >= (1LL << 30)) return MI_EP_EINVAL;
 
   PermuteArgs a{};
   a.x = static_cast<const vec16*>(x);
@@ -313,10 +336,12 @@ int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long lon
   a.xs_hidden_stride = x_scales_hidden_stride;
   a.rs_token_stride = recv_scales_token_stride;
   a.rs_hidden_stride = recv_scales_hidden_stride;
-  hipStream_t s = as_stream(stream);
-  hipError_t e = launch_permute(a, g_permute_schedule.load(std::memory_order_relaxed), s);
-  if (e == hipSuccess && expert_alignment > 1) e = launch_pad_rows(a, expert_alignment, (flags & MI_EP_DISPATCH_KEEP_PAD_PAYLOAD) == 0, s);
-  return status_of(e);
+  a.expert_alignment = expert_alignment;
+  a.zero_pad_payload = (flags & MI_EP_DISPATCH_KEEP_PAD_PAYLOAD) == 0 ? 1 : 0;
+  const int schedule = (flags & MI_EP_DISPATCH_BY_TOKEN) != 0         ? kPermuteByToken
+                       : (flags & MI_EP_DISPATCH_BY_DESTINATION) != 0 ? kPermuteByDestination
+                                                                      : kPermuteAuto;
+  return status_of(launch_permute(a, schedule, as_stream(stream)));
 }
 
 int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
@@ -333,14 +358,17 @@ int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx
                                        recv_topk_weights, slot_map, capacity_rows, flags, stream);
 }
 
-int mi_ep_dispatch_ranks(const void* x, const float* x_scales, const int64_t* topk_idx,
-                         const float* topk_weights, const int* rank_slot_idx, int rank_slot_base,
-                         const int* num_tokens_per_rank, const int* expand_slot_map, int num_tokens,
-                         int num_topk, int num_ranks, int num_experts, int row_bytes, int num_scales,
-                         int source_token_base, int local_expert_ids, void* recv_x, float* recv_scales,
-                         int64_t* recv_topk_idx, float* recv_topk_weights, int* recv_src_metadata,
-                         int* rank_row_map, int* combine_map, int* psum_rank_tokens, int capacity_rows,
-                         void* stream) {
+int mi_ep_dispatch_ranks_strided_scales(const void* x, const float* x_scales, long long x_scales_token_stride,
+                                        long long x_scales_hidden_stride, const int64_t* topk_idx,
+                                        const float* topk_weights, const int* rank_slot_idx, int rank_slot_base,
+                                        const int* num_tokens_per_rank, const int* expand_slot_map,
+                                        int num_tokens, int num_topk, int num_ranks, int num_experts,
+                                        int row_bytes, int num_scales, int source_token_base,
+                                        int local_expert_ids, void* recv_x, float* recv_scales,
+                                        long long recv_scales_token_stride, long long recv_scales_hidden_stride,
+                                        int64_t* recv_topk_idx, float* recv_topk_weights,
+                                        int* recv_src_metadata, int* rank_row_map, int* combine_map,
+                                        int* psum_rank_tokens, int capacity_rows, void* stream) {
   if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
   if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
   if (num_tokens_per_rank == nullptr || psum_rank_tokens == nullptr) return MI_EP_EINVAL;
@@ -351,6 +379,9 @@ int mi_ep_dispatch_ranks(const void* x, const float* x_scales, const int64_t* to
     return MI_EP_EINVAL;
   if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
   if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
+  if (num_scales > 0 && (x_scales_token_stride < 0 || x_scales_hidden_stride < 0 ||
+                         recv_scales_token_stride < 0 || recv_scales_hidden_stride < 0))
+    return MI_EP_EINVAL;
 
   RankPermuteArgs a{};
   a.x = static_cast<const vec16*>(x);
@@ -379,17 +410,39 @@ int mi_ep_dispatch_ranks(const void* x, const float* x_scales, const int64_t* to
   a.rank_slot_base = rank_slot_base;
   a.source_token_base = source_token_base;
   a.local_expert_ids = local_expert_ids != 0;
+  a.xs_token_stride = x_scales_token_stride;
+  a.xs_hidden_stride = x_scales_hidden_stride;
+  a.rs_token_stride = recv_scales_token_stride;
+  a.rs_hidden_stride = recv_scales_hidden_stride;
   return status_of(launch_permute_ranks(a, as_stream(stream)));
 }
 
-int mi_ep_combine_rank_weights(const float* recv_topk_weights, const int* rank_row_map, int num_tokens,
-                               int num_topk, int num_rows, float* combined_topk_weights, void* stream) {
-  if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK || num_rows < 0) return MI_EP_EINVAL;
-  if (static_cast<long long>(num_tokens) * num_topk >= (1LL << 30)) return MI_EP_EINVAL;
-  if (num_tokens > 0 && (rank_row_map == nullptr || combined_topk_weights == nullptr)) return MI_EP_EINVAL;
-  if (num_rows > 0 && recv_topk_weights == nullptr) return MI_EP_EINVAL;
-  return status_of(launch_gather_rank_weights(recv_topk_weights, rank_row_map, num_tokens, num_topk, num_rows,
-                                              combined_topk_weights, as_stream(stream)));
+int mi_ep_dispatch_ranks(const void* x, const float* x_scales, const int64_t* topk_idx,
+                         const float* topk_weights, const int* rank_slot_idx, int rank_slot_base,
+                         const int* num_tokens_per_rank, const int* expand_slot_map, int num_tokens,
+                         int num_topk, int num_ranks, int num_experts, int row_bytes, int num_scales,
+                         int source_token_base, int local_expert_ids, void* recv_x, float* recv_scales,
+                         int64_t* recv_topk_idx, float* recv_topk_weights, int* recv_src_metadata,
+                         int* rank_row_map, int* combine_map, int* psum_rank_tokens, int capacity_rows,
+                         void* stream) {
+  return mi_ep_dispatch_ranks_strided_scales(
+      x, x_scales, num_scales, 1, topk_idx, topk_weights, rank_slot_idx, rank_slot_base, num_tokens_per_rank,
+      expand_slot_map, num_tokens, num_topk, num_ranks, num_experts, row_bytes, num_scales, source_token_base,
+      local_expert_ids, recv_x, recv_scales, num_scales, 1, recv_topk_idx, recv_topk_weights, recv_src_metadata,
+      rank_row_map, combine_map, psum_rank_tokens, capacity_rows, stream);
+}
+
+int mi_ep_combine_rank_weights(const float* recv_topk_weights, const int64_t* recv_topk_idx,
+                               const int* rank_row_map, int num_tokens, int num_topk, int num_rows,
+                               float* combined_topk_weights, int64_t* combined_topk_idx, void* stream) {
+  if (!route_count_ok(num_tokens, num_topk) || num_rows < 0) return MI_EP_EINVAL;
+  if ((recv_topk_weights != nullptr) != (combined_topk_weights != nullptr)) return MI_EP_EINVAL;
+  if ((recv_topk_idx != nullptr) != (combined_topk_idx != nullptr)) return MI_EP_EINVAL;
+  if (combined_topk_weights == nullptr && combined_topk_idx == nullptr) return MI_EP_EINVAL;
+  if (num_tokens > 0 && rank_row_map == nullptr) return MI_EP_EINVAL;
+  return status_of(launch_gather_rank_weights(recv_topk_weights, recv_topk_idx, rank_row_map, num_tokens,
+                                              num_topk, num_rows, combined_topk_weights, combined_topk_idx,
+                                              as_stream(stream)));
 }
 
 int mi_ep_dispatch_cached(const void* x, const float* x_scales, const int* recv_src_map,
@@ -420,12 +473,16 @@ int mi_ep_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_sou
 
 int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
                   const void* bias_0, const void* bias_1, const float* recv_topk_weights,
-                  int num_tokens, int num_topk, int hidden, void* combined_x,
-                  float* combined_topk_weights, void* stream) {
-  if (num_tokens < 0 || num_topk <= 0 || num_topk > MI_EP_MAX_TOPK) return MI_EP_EINVAL;
+                  const int64_t* recv_topk_idx, int num_tokens, int num_topk, int hidden,
+                  void* combined_x, float* combined_topk_weights, int64_t* combined_topk_idx,
+                  void* stream) {
+  if (!route_count_ok(num_tokens, num_topk)) return MI_EP_EINVAL;
   if (hidden <= 0 || hidden % 8 != 0 || num_rows < 0) return MI_EP_EINVAL;
+  // Units of the staged schedule are counted in int: rows of a group times 16-byte vectors.
+  if (static_cast<long long>(hidden) / 8 >= (1LL << 24)) return MI_EP_EINVAL;
   if (num_rows > 0 && y == nullptr) return MI_EP_EINVAL;
   if ((recv_topk_weights != nullptr) != (combined_topk_weights != nullptr)) return MI_EP_EINVAL;
+  if ((recv_topk_idx != nullptr) != (combined_topk_idx != nullptr)) return MI_EP_EINVAL;
   if (num_tokens > 0 && (slot_map == nullptr || combined_x == nullptr)) return MI_EP_EINVAL;
   if (!aligned16(y) || !aligned16(bias_0) || !aligned16(bias_1) || !aligned16(combined_x))
     return MI_EP_EINVAL;
@@ -437,8 +494,10 @@ int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float*
   a.bias_0 = static_cast<const vec16*>(bias_0);
   a.bias_1 = static_cast<const vec16*>(bias_1);
   a.recv_topk_weights = recv_topk_weights;
+  a.recv_topk_idx = recv_topk_idx;
   a.combined_x = static_cast<vec16*>(combined_x);
   a.combined_topk_weights = combined_topk_weights;
+  a.combined_topk_idx = combined_topk_idx;
   a.num_tokens = num_tokens;
   a.num_topk = num_topk;
   a.num_rows = num_rows;

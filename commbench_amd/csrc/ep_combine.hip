@@ -20,6 +20,8 @@
 // Replaces combine_impl + combine_reduce_epilogue_impl (example082 .cu:28-67,
 // example083 .cu:23-53); the reduce buffer of the reference is skipped because
 // the rows already live in this GPU's HBM.
+#include <atomic>
+
 #include "ep_device.h"
 
 namespace mi_ep {
@@ -45,6 +47,8 @@ __device__ __forceinline__ void combine_unit(const CombineArgs& a, const int tok
     if (a.topk_weights != nullptr) weight = a.topk_weights[i];
     if (batch == 0 && a.combined_topk_weights != nullptr)
       a.combined_topk_weights[i] = slot >= 0 ? a.recv_topk_weights[slot] : 0.0f;
+    if (batch == 0 && a.combined_topk_idx != nullptr)
+      a.combined_topk_idx[i] = slot >= 0 ? a.recv_topk_idx[slot] : -1;
   }
   const uint64_t routed = __ballot(slot >= 0);
   const int v0 = batch * (kBatchVecs * kWave) + lane;
@@ -168,24 +172,15 @@ __global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const
   }
 }
 
-int compute_units_of_current_device() {
-  // Cached per device ordinal: a property of the hardware, read once.
-  static int cached[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 template <int kTopk>
 hipError_t launch_combine_k(const CombineArgs& a, hipStream_t stream) {
   const long long row_bytes = static_cast<long long>(a.row_vecs) * 16;
-  const int cus = compute_units_of_current_device();
+  DeviceTraits dev{};
+  int ordinal = 0;
+  hipError_t err = device_traits(stream, &dev);
+  if (err == hipSuccess) err = stream != nullptr ? hipStreamGetDevice(stream, &ordinal) : hipGetDevice(&ordinal);
+  if (err != hipSuccess) return err;
+  const int cus = dev.compute_units;
   // Large shapes: persistent staged schedule.  It needs enough tokens per CU for
   // its phases to be long, and rows that fit the staging area.
   if (a.num_tokens >= 16 * cus && row_bytes >= 2048 && row_bytes <= kStageBytes) {
@@ -198,12 +193,16 @@ hipError_t launch_combine_k(const CombineArgs& a, hipStream_t stream) {
     const int groups = (a.num_tokens + group_tokens - 1) / group_tokens;
     const int grid = groups < cus ? groups : cus;
     const size_t lds = static_cast<size_t>(group_tokens) * row_bytes;
-    static bool lds_limit_raised = false;  // per instantiation; idempotent, so a race is harmless
-    if (!lds_limit_raised) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ep_combine_staged_kernel<kTopk>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes);
+    // The kernel's LDS ceiling is raised once per device (a function attribute lives with the
+    // device's copy of the code object); the flag only ever goes from 0 to 1.
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> lds_limit_raised[kMaxDevices];
+    if (ordinal < 0 || ordinal >= kMaxDevices) return hipErrorInvalidDevice;
+    if (lds_limit_raised[ordinal].load(std::memory_order_acquire) == 0) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ep_combine_staged_kernel<kTopk>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes);
       if (e != hipSuccess) return e;
-      lds_limit_raised = true;
+      lds_limit_raised[ordinal].store(1, std::memory_order_release);
     }
     hipLaunchKernelGGL((ep_combine_staged_kernel<kTopk>), dim3(grid), dim3(kStagedThreads), lds, stream, a,
                        group_tokens);

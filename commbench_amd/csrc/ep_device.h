@@ -28,8 +28,11 @@ constexpr int kChunksPerWave = ((kTileTokens / kWave) * kMaxTopk + kLayoutWaves 
 // {generation + 1, 0}, which is safe because every ticket of the launch is out.
 struct alignas(256) LayoutWorkspace {
   uint64_t turn;
-  uint32_t timed_out;  // sticky: a bounded wait expired
+  uint32_t timed_out;   // sticky: a bounded wait expired
+  uint32_t wait_limit;  // unsuccessful polls before a wait gives up; 0 = kDefaultWaitLimit
 };
+// Polls are spaced by s_sleep, roughly a microsecond apart: a few seconds before a launch gives up.
+constexpr uint32_t kDefaultWaitLimit = 1u << 22;
 
 struct LayoutArgs {
   const int64_t* topk_idx;
@@ -42,6 +45,9 @@ struct LayoutArgs {
   int* slot_rel;
   int* rank_slot_idx;
   int* route_order;  // [num_tiles * kTileTokens * K][4] or null
+  int* tile_rank_counts;         // [num_tiles][R] or null: tokens of the tile flagged for each rank
+  int64_t* copied_topk_idx;      // [T][K] or null: verbatim copy of topk_idx
+  int* cumulative_expert_stats;  // [E] or null: += num_tokens_per_expert
   LayoutWorkspace* ws;
   int* timeout_report;  // null, or a device word that receives MI_EP_ETIMEDOUT when a bounded wait expires
   int num_tokens;
@@ -56,7 +62,6 @@ struct LayoutArgs {
   int expert_bits;  // ceil(log2(num_experts)), at least 1
   uint32_t inv_topk;              // ceil(2^19 / num_topk): n / num_topk == (n * inv) >> 19 for n < 2048
   uint32_t inv_experts_per_rank;  // ceil(2^22 / experts_per_rank): exact for e < 1024
-  uint32_t spin_limit;
 };
 
 hipError_t launch_layout_fused(const LayoutArgs& a, hipStream_t stream);
@@ -92,6 +97,8 @@ struct PermuteArgs {
   // (sf_token_stride / sf_hidden_stride of the reference's dispatch, example080 .cu:40).
   long long xs_token_stride, xs_hidden_stride;
   long long rs_token_stride, rs_hidden_stride;
+  int expert_alignment;  // > 1: segments are padded; the copy kernels also write the pad rows
+  int zero_pad_payload;  // pad rows get zero payload and scales (their map entries are always written)
 };
 
 // Which copy kernel serves mi_ep_dispatch: chosen by shape, or forced (tests, measurements).
@@ -99,15 +106,22 @@ constexpr int kPermuteAuto = 0;
 constexpr int kPermuteByToken = 1;        // wave per (token, 1 KiB): source read once, rows scattered
 constexpr int kPermuteByDestination = 2;  // needs route_order: rows written in destination order
 hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream);
+// What the destination-order copy assumes of the device, read once per device ordinal.
+struct DeviceTraits {
+  int compute_units;  // 256 on the part these kernels are tuned for
+  int dies;           // accelerator dies (XCCs) that take workgroups round-robin
+  int l2_bytes;       // L2 of one die
+};
+// Traits of the device `stream` belongs to (of the current device for the null stream).
+hipError_t device_traits(hipStream_t stream, DeviceTraits* out);
 // The shape rule behind kPermuteAuto (reads num_tokens, num_topk, num_experts, row_vecs only).
-bool destination_order_pays(const PermuteArgs& a);
+bool destination_order_pays(const PermuteArgs& a, const DeviceTraits& dev);
 hipError_t launch_gather_rows(const vec16* x, const float* x_scales, const int* recv_src_map, int num_rows,
                               int num_tokens, int row_vecs, int num_scales, vec16* recv_x,
                               float* recv_scales, int* ready_counters, int rows_per_counter,
                               hipStream_t stream);
 hipError_t launch_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_source_rank,
                                int* pull_indices, hipStream_t stream);
-hipError_t launch_pad_rows(const PermuteArgs& a, int expert_alignment, bool zero_payload, hipStream_t stream);
 
 // Dispatch de-duplicated by destination rank: one row per (token, rank that owns one of its experts).
 struct RankPermuteArgs {
@@ -137,10 +151,14 @@ struct RankPermuteArgs {
   int rank_slot_base;
   int source_token_base;
   int local_expert_ids;
+  // scale factors as [row * token_stride + j * hidden_stride], in 4-byte elements
+  long long xs_token_stride, xs_hidden_stride;
+  long long rs_token_stride, rs_hidden_stride;
 };
 hipError_t launch_permute_ranks(const RankPermuteArgs& a, hipStream_t stream);
-hipError_t launch_gather_rank_weights(const float* recv_topk_weights, const int* rank_row_map, int num_tokens,
-                                      int num_topk, int num_rows, float* combined_topk_weights,
+hipError_t launch_gather_rank_weights(const float* recv_topk_weights, const int64_t* recv_topk_idx,
+                                      const int* rank_row_map, int num_tokens, int num_topk, int num_rows,
+                                      float* combined_topk_weights, int64_t* combined_topk_idx,
                                       hipStream_t stream);
 
 // ---- combine ----------------------------------------------------------------
@@ -151,8 +169,10 @@ struct CombineArgs {
   const vec16* bias_0;
   const vec16* bias_1;
   const float* recv_topk_weights;
+  const int64_t* recv_topk_idx;
   vec16* combined_x;
   float* combined_topk_weights;
+  int64_t* combined_topk_idx;
   int num_tokens;
   int num_topk;
   int num_rows;  // rows of y; map entries at or beyond it are treated as non-routes

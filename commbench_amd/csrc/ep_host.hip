@@ -89,6 +89,73 @@ int mi_ep_host_get_dispatch_layout(const int64_t* topk_idx, int* num_tokens_per_
   return s.status(MI_EP_OK);
 }
 
+int mi_ep_host_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
+                               int num_experts, int expert_alignment, int num_channels,
+                               int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
+                               int* expert_offsets, int* psum_rank_rows, int* channel_prefix_matrix,
+                               int* slot_rel, int* rank_slot_idx, int rank_slot_base, int* route_order,
+                               int* tile_rank_counts, int64_t* copied_topk_idx, int* cumulative_expert_stats) {
+  if (num_tokens < 0 || num_topk <= 0 || num_ranks <= 0 || num_experts <= 0 || expert_alignment < 1)
+    return MI_EP_EINVAL;
+  if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
+  if (num_tokens > 0 && (topk_idx == nullptr || is_token_in_rank == nullptr)) return MI_EP_EINVAL;
+  if (channel_prefix_matrix != nullptr && num_channels < 1) return MI_EP_EINVAL;
+  const size_t workspace_bytes = mi_ep_workspace_bytes(num_tokens > 0 ? num_tokens : 1, num_topk, num_experts, num_ranks);
+  if (workspace_bytes == 0) return MI_EP_EINVAL;
+
+  Staging s;
+  const size_t tk = static_cast<size_t>(num_tokens) * num_topk;
+  const size_t tr = static_cast<size_t>(num_tokens) * num_ranks;
+  const size_t tiles = (static_cast<size_t>(num_tokens) + 255) / 256;
+  const size_t order_ints = mi_ep_route_order_bytes(num_tokens, num_topk) / sizeof(int);
+  const size_t rc = channel_prefix_matrix != nullptr ? static_cast<size_t>(num_ranks) * num_channels : 0;
+  const int64_t* d_topk = s.upload(topk_idx, tk);
+  int* d_rank = s.alloc<int>(num_ranks);
+  int* d_expert = s.alloc<int>(num_experts);
+  bool* d_flags = s.alloc<bool>(tr);
+  int* d_off = expert_offsets != nullptr ? s.alloc<int>(static_cast<size_t>(num_experts) + 1) : nullptr;
+  int* d_psum = psum_rank_rows != nullptr ? s.alloc<int>(num_ranks) : nullptr;
+  int* d_prefix = channel_prefix_matrix != nullptr ? s.alloc<int>(rc) : nullptr;
+  int* d_slot_rel = slot_rel != nullptr ? s.alloc<int>(tk) : nullptr;
+  int* d_rank_slots = rank_slot_idx != nullptr ? s.alloc<int>(tk) : nullptr;
+  int* d_order = route_order != nullptr ? s.alloc<int>(order_ints) : nullptr;
+  int* d_tile_ranks = tile_rank_counts != nullptr ? s.alloc<int>(tiles * num_ranks) : nullptr;
+  int64_t* d_copied = copied_topk_idx != nullptr ? s.alloc<int64_t>(tk) : nullptr;
+  // The running statistics continue from the caller's values.
+  int* d_stats = cumulative_expert_stats != nullptr
+                     ? const_cast<int*>(s.upload(static_cast<const int*>(cumulative_expert_stats), num_experts))
+                     : nullptr;
+  unsigned char* d_ws = s.alloc<unsigned char>(workspace_bytes);
+  if (!s.ok()) return s.status(MI_EP_OK);
+  if (d_order != nullptr && order_ints > 0) {
+    // Entries past the last token are not written by the kernel: hand back zeros there.
+    s.err = hipMemset(d_order, 0, order_ints * sizeof(int));
+    if (!s.ok()) return s.status(MI_EP_OK);
+  }
+
+  int code = mi_ep_workspace_init(d_ws, workspace_bytes, nullptr);
+  if (code == MI_EP_OK)
+    code = mi_ep_dispatch_layout(d_topk, num_tokens, num_topk, num_ranks, num_experts, expert_alignment,
+                                 num_channels, d_rank, d_expert, d_flags, d_off, d_psum, d_prefix, d_slot_rel,
+                                 d_rank_slots, rank_slot_base, d_order, d_tile_ranks, d_copied, d_stats, d_ws,
+                                 workspace_bytes, nullptr);
+  if (code == MI_EP_OK) code = mi_ep_workspace_status(d_ws, nullptr);  // synchronises
+  if (code != MI_EP_OK) return code;
+  s.download(num_tokens_per_rank, d_rank, num_ranks);
+  s.download(num_tokens_per_expert, d_expert, num_experts);
+  s.download(is_token_in_rank, d_flags, tr);
+  s.download(expert_offsets, d_off, static_cast<size_t>(num_experts) + 1);
+  s.download(psum_rank_rows, d_psum, num_ranks);
+  s.download(channel_prefix_matrix, d_prefix, rc);
+  s.download(slot_rel, d_slot_rel, tk);
+  s.download(rank_slot_idx, d_rank_slots, tk);
+  s.download(route_order, d_order, order_ints);
+  s.download(tile_rank_counts, d_tile_ranks, tiles * num_ranks);
+  s.download(copied_topk_idx, d_copied, tk);
+  s.download(cumulative_expert_stats, d_stats, num_experts);
+  return s.status(MI_EP_OK);
+}
+
 int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
                         const float* topk_weights, int num_tokens, int num_topk, int num_ranks,
                         int num_experts, int expert_alignment, int row_bytes, int num_scales,
@@ -134,7 +201,7 @@ int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* top
   if (code == MI_EP_OK)
     code = mi_ep_dispatch_layout(d_topk, num_tokens, num_topk, num_ranks, num_experts, expert_alignment, 0,
                                  d_rank, d_expert, d_flags, d_off, nullptr, nullptr, d_slot_rel, nullptr, 0,
-                                 d_order, d_ws, workspace_bytes, nullptr);
+                                 d_order, nullptr, nullptr, nullptr, d_ws, workspace_bytes, nullptr);
   if (code == MI_EP_OK)
     code = mi_ep_dispatch(d_x, d_scales, d_topk, d_w, d_off, d_slot_rel, d_order, d_expert, num_tokens,
                           num_topk, num_experts, expert_alignment, row_bytes, num_scales, d_recv_x,
@@ -175,8 +242,8 @@ int mi_ep_host_combine(const void* y, int num_rows, const int* slot_map, const f
   const uint16_t* d_b1 = s.upload(static_cast<const uint16_t*>(bias_1), th);
   uint16_t* d_out = s.alloc<uint16_t>(th);
   if (!s.ok()) return s.status(MI_EP_OK);
-  int code = mi_ep_combine(d_y, num_rows, d_map, d_w, d_b0, d_b1, nullptr, num_tokens, num_topk, hidden,
-                           d_out, nullptr, nullptr);
+  int code = mi_ep_combine(d_y, num_rows, d_map, d_w, d_b0, d_b1, nullptr, nullptr, num_tokens, num_topk,
+                           hidden, d_out, nullptr, nullptr, nullptr);
   code = sync_status(code);
   if (code != MI_EP_OK) return code;
   s.download(static_cast<uint16_t*>(combined_x), d_out, th);

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   int* col_excl = col_total + cols;         // [cols] sum over earlier tiles
   int* rank_cnt = col_excl + cols;          // [kMaxRanks]
   int* wave_sums = rank_cnt + kMaxRanks;    // [kLayoutWaves]
-  int* misc = wave_sums + kLayoutWaves;     // [4] tile, generation
+  int* misc = wave_sums + kLayoutWaves;     // [4] tile, generation, wait limit
   int* rank_wave = misc + 4;                // [kTileTokens / kWave][kMaxRanks] flagged tokens per wave
   int* order_sums = rank_wave + (kTileTokens / kWave) * kMaxRanks;  // [kLayoutWaves] scan of the tile's counts
   int* masked_wave = order_sums + kLayoutWaves;                      // [kLayoutWaves] non-routes per wave
@@ -105,6 +105,8 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     const uint32_t generation = static_cast<uint32_t>(turn >> 32) & kGenMask;
     misc[0] = static_cast<int>(ticket);
     misc[1] = static_cast<int>(generation);
+    const uint32_t limit = a.ws->wait_limit;
+    misc[2] = static_cast<int>(limit != 0 ? limit : kDefaultWaitLimit);
     // Last ticket of the launch: hand the workspace to the next launch.
     if (ticket == static_cast<uint32_t>(a.num_tiles) - 1u)
       __hip_atomic_store(&a.ws->turn, static_cast<uint64_t>((generation + 1u) & kGenMask) << 32,
@@ -120,6 +122,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
 
   const int tile = misc[0];
   const uint32_t gen = static_cast<uint32_t>(misc[1]);
+  const uint32_t wait_limit = static_cast<uint32_t>(misc[2]);
   if (tile >= a.num_tiles) return;  // stale ticket: never with an initialised workspace
   const int t0 = tile * kTileTokens;
   const int flat0 = t0 * K;
@@ -137,7 +140,10 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     const int chunk = wave * per_wave + c;
     if (c < per_wave && chunk < num_chunks) {
       const int g = flat0 + chunk * kWave + lane;
-      if (g < flat_end) raw[c] = a.topk_idx[g];
+      if (g < flat_end) {
+        raw[c] = a.topk_idx[g];
+        if (a.copied_topk_idx != nullptr) a.copied_topk_idx[g] = raw[c];
+      }
     }
   }
   int my_e[kChunksPerWave];
@@ -239,6 +245,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     } else {
       total = rank_cnt[col - E];
       col_total[col] = total;
+      if (a.tile_rank_counts != nullptr) a.tile_rank_counts[static_cast<size_t>(tile) * R + (col - E)] = total;
       publish(mine, pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
     }
     int excl = 0;
@@ -273,7 +280,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
           }
         }
         if (stalled) {
-          if (++spins >= a.spin_limit) {
+          if (++spins >= wait_limit) {
             __hip_atomic_store(&a.ws->timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (a.timeout_report != nullptr)
               __hip_atomic_store(a.timeout_report, kTimedOutCode, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -378,10 +385,13 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   if (tile == a.num_tiles - 1) {
     for (int col = tid; col < cols; col += kLayoutThreads) {
       const int cnt = col_excl[col] + col_total[col];
-      if (col < E)
+      if (col < E) {
         a.num_tokens_per_expert[col] = cnt;
-      else
+        // One adder per launch and expert; launches that share the array may overlap, hence atomic.
+        if (a.cumulative_expert_stats != nullptr && cnt != 0) atomicAdd(&a.cumulative_expert_stats[col], cnt);
+      } else {
         a.num_tokens_per_rank[col - E] = cnt;
+      }
     }
     if (a.expert_offsets != nullptr) {
       // Block-wide exclusive scan of the aligned counts, one expert per thread

@@ -4,7 +4,8 @@
 //   ep_permute_tiles_kernel   destination order, for long rows on large batches (further down)
 //   ep_permute_kernel         token order, everything else
 //   ep_permute_ranks_kernel   one row per (token, destination rank), the reference's own format
-// plus the pad-row fill, the pull-mode gathers and the bandwidth yardsticks.
+// plus the pull-mode gathers and the bandwidth yardsticks.  With expert_alignment > 1 the first two
+// also write the pad rows of every segment from extra units of the same launch.
 //
 // ep_permute_kernel: each wavefront owns (token, batch): one batch is up to
 // kBatchVecs * 64 consecutive 16-byte vectors of the token's row (1 KiB as launched).  The wave reads
@@ -16,6 +17,8 @@
 // Replaces the payload role of dispatch_impl (example080 .cu:241-256) and the
 // expand-mode copy epilogue (example081 .cu:22-60); one partition of this GPU's
 // HBM stands where the reference has a peer GPU's receive buffer.
+#include <atomic>
+
 #include "ep_device.h"
 
 namespace mi_ep {
@@ -28,16 +31,56 @@ constexpr int kPermuteWaves = kPermuteThreads / kWave;
 // occupancy, and finer units even out the tail.
 constexpr int kPushThreads = 128;
 constexpr int kPushWaves = kPushThreads / kWave;
-// The destination-order kernel leans on two facts of this GPU: eight accelerator dies that take
-// workgroups round-robin, each with a 4 MiB L2.  A tile's source rows must fit that L2 with room
-// for the routing tables.
+// The destination-order kernel leans on two facts of the GPU it was tuned on: eight accelerator
+// dies that take workgroups round-robin, each with a 4 MiB L2.  A tile's source rows must fit that
+// L2 with room for the routing tables; on a device that reports anything else (another partition
+// mode, another part) the token-order kernel is used.
 constexpr int kDies = 8;
+constexpr int kDieL2BytesMin = 4 * 1024 * 1024;
 constexpr size_t kTileSourceBytesMax = 3840u * 1024u;
 constexpr size_t kRowBytesMin = 4u * 1024u;
 constexpr size_t kFatRowBytesMax = 12u * 1024u;  // below this, 8 KiB instead of 2 KiB per workgroup
 constexpr int kRunRowsMin = 4;
 // The first workgroups of a tile pull its source rows into L2, 8 rows per group of workgroups.
 constexpr int kPrefetchGroups = 32;
+
+
+// The same pointer in the constant address space: for memory that no thread of the launch writes.
+template <typename T>
+__device__ __forceinline__ const T __attribute__((address_space(4)))* as_constant(const T* p) {
+  return reinterpret_cast<const T __attribute__((address_space(4)))*>(reinterpret_cast<uintptr_t>(p));
+}
+
+// Pad rows (expert_alignment > 1): item p stands for possible pad row i = p % (align - 1) of expert
+// e = p / (align - 1); it exists when off[e] + count[e] + i is still inside the padded segment and
+// the capacity.  Returns the row, or -1.
+__device__ __forceinline__ int pad_row_of_item(const PermuteArgs& a, const int item) {
+  const int per_expert = a.expert_alignment - 1;
+  const int e = item / per_expert;
+  if (e >= a.num_experts) return -1;
+  const int i = item - e * per_expert;
+  const int begin = a.expert_offsets[e] + a.num_tokens_per_expert[e];
+  int end = a.expert_offsets[e + 1];
+  if (end > a.capacity_rows) end = a.capacity_rows;
+  const int row = begin + i;
+  return (begin >= 0 && row < end) ? row : -1;
+}
+
+// Side data of the pad rows, one item per thread: source -1, expert -1, weight 0, and zero scale
+// factors when the payload is zeroed too.  Called by `threads` threads numbered `first`...
+__device__ __forceinline__ void write_pad_markers(const PermuteArgs& a, const long long first, const long long threads) {
+  const long long items = static_cast<long long>(a.num_experts) * (a.expert_alignment - 1);
+  for (long long item = first; item < items; item += threads) {
+    const int row = pad_row_of_item(a, static_cast<int>(item));
+    if (row < 0) continue;
+    a.recv_src_map[row] = -1;
+    if (a.recv_topk_idx != nullptr) a.recv_topk_idx[row] = -1;
+    if (a.recv_topk_weights != nullptr) a.recv_topk_weights[row] = 0.0f;
+    if (a.zero_pad_payload && a.recv_scales != nullptr)
+      for (int j = 0; j < a.num_scales; ++j)
+        a.recv_scales[static_cast<size_t>(row) * a.rs_token_stride + static_cast<size_t>(j) * a.rs_hidden_stride] = 0.0f;
+  }
+}
 
 template <int kBatchVecs, bool kStreamStores>
 __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteArgs a,
@@ -47,7 +90,33 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
   const long long unit = static_cast<long long>(blockIdx.x) * kPushWaves + wave;
   const int token = static_cast<int>(unit / batches_per_row);
   const int batch = static_cast<int>(unit - static_cast<long long>(token) * batches_per_row);
-  if (token >= a.num_tokens) return;
+  if (token >= a.num_tokens) {
+    if (a.expert_alignment <= 1) return;
+    // Units past the last token: first the pad rows' side data (one item per lane), then, when the
+    // pads are zeroed, one unit per (pad item, batch) in row order, so that the fill is a linear
+    // stream wherever pad rows are adjacent.
+    const long long items = static_cast<long long>(a.num_experts) * (a.expert_alignment - 1);
+    const long long marker_units = (items + kWave - 1) / kWave;
+    const long long u = unit - static_cast<long long>(a.num_tokens) * batches_per_row;
+    if (u < marker_units) {
+      write_pad_markers(a, u * kWave + lane, marker_units * kWave);
+      return;
+    }
+    if (!a.zero_pad_payload) return;
+    const long long z = u - marker_units;
+    const long long item = z / batches_per_row;
+    if (item >= items) return;
+    const int row = pad_row_of_item(a, static_cast<int>(item));
+    if (row < 0) return;
+    const int zb = static_cast<int>(z - item * batches_per_row);
+    const vec16 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int q = 0; q < kBatchVecs; ++q) {
+      const int v = zb * (kBatchVecs * kWave) + q * kWave + lane;
+      if (v < a.row_vecs) __builtin_nontemporal_store(zero, a.recv_x + static_cast<size_t>(row) * a.row_vecs + v);
+    }
+    return;
+  }
   const int K = a.num_topk;
 
   // Payload loads first: they do not depend on the routing data.
@@ -69,7 +138,8 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
     expert = a.topk_idx[i];
     if (rel >= 0 && expert >= 0 && expert < static_cast<int64_t>(a.num_experts)) {
       slot = a.expert_offsets[expert] + rel;
-      if (slot >= a.capacity_rows) slot = -1;
+      // beyond the capacity, or tables that are not a finished layout's: dropped, never written
+      if (slot < 0 || slot >= a.capacity_rows) slot = -1;
     }
     if (batch == 0) {
       a.slot_map[i] = slot;
@@ -115,6 +185,15 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
   }
 }
 
+// The prefetch workgroups of the destination-order kernel (of every die and round, also those
+// without a tile) share out the pad rows' side data, one item per thread.
+__device__ __forceinline__ void pad_markers_from_prefetch_workgroup(const PermuteArgs& a, const int prefetch_ys,
+                                                                    const int rounds) {
+  const long long wg = (static_cast<long long>(blockIdx.z) * prefetch_ys + blockIdx.y) * gridDim.x + blockIdx.x;
+  write_pad_markers(a, wg * kPushThreads + static_cast<int>(threadIdx.x),
+                    static_cast<long long>(rounds) * prefetch_ys * gridDim.x * kPushThreads);
+}
+
 // The same copy in destination order.  A tile is the layout kernel's 256 tokens; its
 // routes arrive sorted by (expert, position in segment), so consecutive workgroups write
 // consecutive rows of recv_x: a tile leaves ~256*K/E adjacent rows per expert, which the
@@ -127,34 +206,63 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
 // Launched as a 3-D grid (x = part of the row * 8 + die, y = entry of the tile's list, z = round
 // of eight tiles) so that no index needs a division: a wave moves only 1 KiB, which leaves it
 // a budget of about a hundred vector instructions before instruction issue, not HBM, sets the pace.
-template <bool kStreamStores, int kVecs>
+// kPads: expert_alignment > 1 (pad markers and pad rounds compiled in); kScales: scale factors travel.
+template <int kVecs, bool kPads, bool kScales>
 __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const PermuteArgs a, const int num_tiles,
-                                                                       const int prefetch_ys) {
+                                                                       const int rounds) {
+  constexpr int prefetch_ys = kPrefetchGroups;
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
   const int die = static_cast<int>(blockIdx.x) & (kDies - 1);
   const int part = static_cast<int>(blockIdx.x) >> 3;
   const int tile = static_cast<int>(blockIdx.z) * kDies + die;
-  if (tile >= num_tiles) return;
+  // Everything that is not a route copy returns before the copy's code: pad rounds and dies without
+  // a tile in the last round first, then the tile's prefetch workgroups.
+  if (tile >= num_tiles) {
+    if (!kPads) return;
+    if (static_cast<int>(blockIdx.z) >= rounds) {
+      // Pad rounds (only launched when pad rows are zeroed): workgroup (die, y) of pad round r takes
+      // pad item ((r * gridDim.y + y) * 8 + die), so the dies write adjacent rows side by side.
+      const long long item = (static_cast<long long>(static_cast<int>(blockIdx.z) - rounds) * gridDim.y + blockIdx.y) * kDies + die;
+      if (item >= static_cast<long long>(a.num_experts) * (a.expert_alignment - 1)) return;
+      const int row = pad_row_of_item(a, static_cast<int>(item));
+      if (row < 0) return;
+      const vec16 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int u = 0; u < kVecs; ++u) {
+        const int v = (part * kPushWaves + wave) * (kWave * kVecs) + u * kWave + lane;
+        if (v < a.row_vecs) __builtin_nontemporal_store(zero, a.recv_x + static_cast<size_t>(row) * a.row_vecs + v);
+      }
+      return;
+    }
+    if (static_cast<int>(blockIdx.y) < prefetch_ys) pad_markers_from_prefetch_workgroup(a, prefetch_ys, rounds);
+    return;
+  }
   if (static_cast<int>(blockIdx.y) < prefetch_ys) {
+    if (kPads) pad_markers_from_prefetch_workgroup(a, prefetch_ys, rounds);
     // The tile's first workgroups pull its source rows into the die's L2 as one linear burst:
     // when the rows come from HBM (not from the memory-side cache) this keeps their reads from
     // being sprinkled over the whole tile, where they would break up the runs of writes
-    // (measured at 8192 x 14 KiB rows: 182 us against 208 us; 2-3 us lost when the rows are cached).
+    // (measured at 8192 x 14 KiB rows: 182 us against 208 us; a few us lost when the rows are cached).
     const int v0 = (part * kPushWaves + wave) * (kWave * kVecs) + lane;
-    const int rows_per_y = kTileTokens / prefetch_ys;
+    constexpr int rows_per_y = kTileTokens / prefetch_ys;
     const int row0 = tile * kTileTokens + static_cast<int>(blockIdx.y) * rows_per_y;
+    // Rows past the last token are clamped to it, so that all loads are issued back to back under
+    // one condition and the workgroup lives for one memory round trip, not eight.
     uint32_t fold = 0;
-    for (int i = 0; i < rows_per_y; ++i) {
-      if (row0 + i < a.num_tokens) {
+    const int last_row = a.num_tokens - 1;
 #pragma unroll
-        for (int u = 0; u < kVecs; ++u) {
-          const int v = v0 + u * kWave;
-          if (v < a.row_vecs) {
-            const vec16 q = a.x[static_cast<size_t>(row0 + i) * a.row_vecs + v];
-            fold ^= q[0] ^ q[1] ^ q[2] ^ q[3];
-          }
+    for (int u = 0; u < kVecs; ++u) {
+      const int v = v0 + u * kWave;
+      if (v < a.row_vecs) {
+        vec16 q[rows_per_y];
+#pragma unroll
+        for (int i = 0; i < rows_per_y; ++i) {
+          const int row = row0 + i < last_row ? row0 + i : last_row;
+          q[i] = a.x[static_cast<size_t>(row) * a.row_vecs + v];
         }
+#pragma unroll
+        for (int i = 0; i < rows_per_y; ++i) fold ^= q[i][0] ^ q[i][1] ^ q[i][2] ^ q[i][3];
       }
     }
     if (fold == 0x9e3779b9u && a.capacity_rows < 0) a.slot_map[0] = -1;  // never true: keeps the loads alive
@@ -166,11 +274,15 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
   const int routes = (tokens_left < kTileTokens ? tokens_left : kTileTokens) * K;
   if (entry >= routes) return;
   const int first_flat = tile * kTileTokens * K;
-  const int4 r = reinterpret_cast<const int4*>(a.route_order)[static_cast<size_t>(first_flat) + entry];
-  const int flat = __builtin_amdgcn_readfirstlane(r.x);
-  const int expert = __builtin_amdgcn_readfirstlane(r.y);
-  const int rel = __builtin_amdgcn_readfirstlane(r.z);
-  const int token = __builtin_amdgcn_readfirstlane(r.w);
+  // The routing tables are only read here: through the constant address space their (wave-uniform)
+  // loads are scalar loads whatever else the kernel stores.
+  typedef int route_entry __attribute__((ext_vector_type(4)));
+  const route_entry r =
+      as_constant(reinterpret_cast<const route_entry*>(a.route_order))[static_cast<size_t>(first_flat) + entry];
+  const int flat = __builtin_amdgcn_readfirstlane(r[0]);
+  const int expert = __builtin_amdgcn_readfirstlane(r[1]);
+  const int rel = __builtin_amdgcn_readfirstlane(r[2]);
+  const int token = __builtin_amdgcn_readfirstlane(r[3]);
   // A table that is not this launch's (wrong shape, stale memory) must not send accesses astray.
   if (flat < first_flat || flat >= first_flat + routes || token < 0 || token >= a.num_tokens) return;
   const bool routed = expert >= 0 && expert < a.num_experts && rel >= 0;
@@ -185,8 +297,8 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
 
   int slot = -1;
   if (routed) {
-    slot = a.expert_offsets[expert] + rel;
-    if (slot >= a.capacity_rows) slot = -1;
+    slot = as_constant(a.expert_offsets)[expert] + rel;
+    if (slot < 0 || slot >= a.capacity_rows) slot = -1;
   }
   if (part == 0 && wave == 0) {
     if (lane == 0) {
@@ -198,7 +310,7 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
           a.recv_topk_weights[slot] = a.topk_weights != nullptr ? a.topk_weights[flat] : 1.0f;
       }
     }
-    if (slot >= 0 && a.recv_scales != nullptr)
+    if (kScales && slot >= 0)
       for (int j = lane; j < a.num_scales; j += kWave)
         a.recv_scales[static_cast<size_t>(slot) * a.rs_token_stride + static_cast<size_t>(j) * a.rs_hidden_stride] =
             a.x_scales[static_cast<size_t>(token) * a.xs_token_stride + static_cast<size_t>(j) * a.xs_hidden_stride];
@@ -207,15 +319,25 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
 #pragma unroll
     for (int u = 0; u < kVecs; ++u) {
       const int v = v0 + u * kWave;
-      if (v < a.row_vecs) {
-        vec16* dst = a.recv_x + static_cast<size_t>(slot) * a.row_vecs + v;
-        if (kStreamStores)
-          __builtin_nontemporal_store(buf[u], dst);
-        else
-          *dst = buf[u];
-      }
+      if (v < a.row_vecs)
+        __builtin_nontemporal_store(buf[u], a.recv_x + static_cast<size_t>(slot) * a.row_vecs + v);
     }
   }
+}
+
+template <int kVecs>
+hipError_t launch_permute_tiles(const PermuteArgs& a, const dim3 grid, const int tiles, const int rounds,
+                                hipStream_t stream) {
+  const bool pads = a.expert_alignment > 1, scales = a.recv_scales != nullptr;
+  if (pads && scales)
+    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, true, true>), grid, dim3(kPushThreads), 0, stream, a, tiles, rounds);
+  else if (pads)
+    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, true, false>), grid, dim3(kPushThreads), 0, stream, a, tiles, rounds);
+  else if (scales)
+    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, false, true>), grid, dim3(kPushThreads), 0, stream, a, tiles, rounds);
+  else
+    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, false, false>), grid, dim3(kPushThreads), 0, stream, a, tiles, rounds);
+  return hipGetLastError();
 }
 
 // Dispatch de-duplicated by destination rank (the reference's own format: payload role of
@@ -243,6 +365,16 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_ranks_kernel(const Ra
   vec16 buf = {0u, 0u, 0u, 0u};
   if (v < a.row_vecs) buf = src[v];
 
+  // First row of every rank: an exclusive scan of the layout's per-rank counts (at most 8 of them).
+  int rank_base[kMaxRanks];
+  {
+    int run = 0;
+#pragma unroll
+    for (int r = 0; r < kMaxRanks; ++r) {
+      rank_base[r] = run;
+      if (r < a.num_ranks) run += a.num_tokens_per_rank[r];  // wave-uniform addresses: scalar loads
+    }
+  }
   // Lane k < K resolves slot k: its rank, and on the first slot of a rank the row it opens.
   const size_t i = static_cast<size_t>(token) * K + (lane < K ? lane : 0);
   int64_t expert = -1;
@@ -255,9 +387,7 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_ranks_kernel(const Ra
       const int slot = a.rank_slot_idx[i];
       opens = slot >= 0;
       if (opens) {
-        int base = 0;
-        for (int r = 0; r < rank; ++r) base += a.num_tokens_per_rank[r];
-        own_row = base + (slot - a.rank_slot_base);
+        own_row = rank_base[rank] + (slot - a.rank_slot_base);
         if (own_row < 0 || own_row >= a.capacity_rows) own_row = -1;  // dropped
       }
     }
@@ -299,8 +429,8 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_ranks_kernel(const Ra
       }
       if (a.recv_scales != nullptr)
         for (int s = lane; s < a.num_scales; s += kWave)
-          a.recv_scales[static_cast<size_t>(row) * a.num_scales + s] =
-              a.x_scales[static_cast<size_t>(token) * a.num_scales + s];
+          a.recv_scales[static_cast<size_t>(row) * a.rs_token_stride + static_cast<size_t>(s) * a.rs_hidden_stride] =
+              a.x_scales[static_cast<size_t>(token) * a.xs_token_stride + static_cast<size_t>(s) * a.xs_hidden_stride];
     }
   }
 
@@ -314,44 +444,23 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_ranks_kernel(const Ra
   }
 }
 
-// combined_topk_weights[t,k] = the weight that travelled with route (t,k) in the per-rank format.
+// combined_topk_weights[t,k] / combined_topk_idx[t,k] = the weight / expert id that travelled with
+// route (t,k) in the per-rank format (0 / -1 for non-routes).
 __global__ __launch_bounds__(256) void ep_gather_rank_weights_kernel(const float* __restrict__ recv_topk_weights,
+                                                                    const int64_t* __restrict__ recv_topk_idx,
                                                                     const int* __restrict__ rank_row_map,
                                                                     const int total, const int num_topk,
                                                                     const int num_rows,
-                                                                    float* __restrict__ out) {
+                                                                    float* __restrict__ out_weights,
+                                                                    int64_t* __restrict__ out_idx) {
   const int i = static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
   if (i >= total) return;
   const int row = rank_row_map[i];
   const int k = i % num_topk;
-  out[i] = (row >= 0 && row < num_rows) ? recv_topk_weights[static_cast<size_t>(row) * num_topk + k] : 0.0f;
-}
-
-// Zero-fills the rows that expert_alignment > 1 leaves between a segment's last
-// route and the next segment.  Workgroup (e, j) takes pad rows j, j + gridDim.y, ... of
-// expert e: at alignment 128 the pads are a fifth of the buffer, so they are spread over
-// the whole device rather than walked by one workgroup per expert.
-__global__ __launch_bounds__(kPermuteThreads) void ep_pad_rows_kernel(const PermuteArgs a, const bool zero_payload) {
-  const int e = static_cast<int>(blockIdx.x);
-  const int begin = a.expert_offsets[e] + a.num_tokens_per_expert[e];
-  int end = a.expert_offsets[e + 1];
-  if (end > a.capacity_rows) end = a.capacity_rows;
-  const int tid = static_cast<int>(threadIdx.x);
-  const vec16 zero = {0u, 0u, 0u, 0u};
-  for (int row = begin + static_cast<int>(blockIdx.y); row < end; row += static_cast<int>(gridDim.y)) {
-    if (zero_payload) {
-      vec16* dst = a.recv_x + static_cast<size_t>(row) * a.row_vecs;
-      for (int v = tid; v < a.row_vecs; v += kPermuteThreads) __builtin_nontemporal_store(zero, dst + v);
-      if (a.recv_scales != nullptr)
-        for (int j = tid; j < a.num_scales; j += kPermuteThreads)
-          a.recv_scales[static_cast<size_t>(row) * a.rs_token_stride + static_cast<size_t>(j) * a.rs_hidden_stride] = 0.0f;
-    }
-    if (tid == 0) {
-      a.recv_src_map[row] = -1;
-      if (a.recv_topk_idx != nullptr) a.recv_topk_idx[row] = -1;
-      if (a.recv_topk_weights != nullptr) a.recv_topk_weights[row] = 0.0f;
-    }
-  }
+  const bool live = row >= 0 && row < num_rows;
+  if (out_weights != nullptr)
+    out_weights[i] = live ? recv_topk_weights[static_cast<size_t>(row) * num_topk + k] : 0.0f;
+  if (out_idx != nullptr) out_idx[i] = live ? recv_topk_idx[static_cast<size_t>(row) * num_topk + k] : -1;
 }
 
 // Pull-mode dispatch: one wave per (destination row, batch).  Destination rows are
@@ -489,7 +598,34 @@ __global__ __launch_bounds__(256) void ep_write_yardstick_kernel(vec16* __restri
 // rows are long enough for a workgroup to have something to move and a tile leaves an expert a
 // run of several adjacent rows.  Measured against the token-major kernel, whole copy:
 // 14 KiB rows -13..-16 %, 8 KiB rows -8..-13 %, 4 KiB rows -13 %, 6-7 KiB rows -3..0 %.
-bool destination_order_pays(const PermuteArgs& a) {
+hipError_t device_traits(hipStream_t stream, DeviceTraits* out) {
+  // Properties of the hardware, read once per device ordinal and never changed afterwards.
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> ready[kMaxDevices];
+  static DeviceTraits cached[kMaxDevices];
+  int dev = 0;
+  hipError_t e = stream != nullptr ? hipStreamGetDevice(stream, &dev) : hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  if (ready[dev].load(std::memory_order_acquire) == 0) {
+    DeviceTraits t{};
+    if (hipDeviceGetAttribute(&t.compute_units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        t.compute_units <= 0)
+      t.compute_units = 256;
+    // Unknown values (an attribute this runtime does not report) switch the destination order off.
+    if (hipDeviceGetAttribute(&t.dies, hipDeviceAttributeNumberOfXccs, dev) != hipSuccess) t.dies = 0;
+    if (hipDeviceGetAttribute(&t.l2_bytes, hipDeviceAttributeL2CacheSize, dev) != hipSuccess) t.l2_bytes = 0;
+    (void)hipGetLastError();
+    cached[dev] = t;  // racing first calls store the same values
+    ready[dev].store(1, std::memory_order_release);
+  }
+  *out = cached[dev];
+  return hipSuccess;
+}
+
+bool destination_order_pays(const PermuteArgs& a, const DeviceTraits& dev) {
+  // The die mapping and the L2 budget are built into the kernel: any other device takes the token order.
+  if (dev.dies != kDies || dev.l2_bytes < kDieL2BytesMin) return false;
   const int tiles = (a.num_tokens + kTileTokens - 1) / kTileTokens;
   const int rounds = (tiles + kDies - 1) / kDies;
   if (tiles * 8 < rounds * kDies * 7) return false;  // more than 1/8 of the die-rounds idle
@@ -500,10 +636,15 @@ bool destination_order_pays(const PermuteArgs& a) {
 }
 
 hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream) {
-  if (a.num_tokens == 0) return hipSuccess;
-  const bool by_destination =
-      a.route_order != nullptr && (schedule == kPermuteByDestination ||
-                                   (schedule == kPermuteAuto && destination_order_pays(a)));
+  const long long pad_items = a.expert_alignment > 1 ? static_cast<long long>(a.num_experts) * (a.expert_alignment - 1) : 0;
+  if (a.num_tokens == 0 && pad_items == 0) return hipSuccess;
+  bool by_destination = a.num_tokens > 0 && a.route_order != nullptr && schedule == kPermuteByDestination;
+  if (a.num_tokens > 0 && a.route_order != nullptr && schedule == kPermuteAuto) {
+    DeviceTraits dev{};
+    const hipError_t e = device_traits(stream, &dev);
+    if (e != hipSuccess) return e;
+    by_destination = destination_order_pays(a, dev);
+  }
   if (by_destination) {
     const int tiles = (a.num_tokens + kTileTokens - 1) / kTileTokens;
     const int rounds = (tiles + kDies - 1) / kDies;
@@ -512,21 +653,23 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
     const bool fat = static_cast<size_t>(a.row_vecs) * sizeof(vec16) < kFatRowBytesMax;
     const int per_workgroup = kPushWaves * kWave * (fat ? 4 : 1);
     const int parts = (a.row_vecs + per_workgroup - 1) / per_workgroup;
-    if (rounds > 65535 || parts * kDies > 65535) return hipErrorInvalidValue;
     const int prefetch_ys = kPrefetchGroups;
-    const dim3 grid(static_cast<unsigned>(parts * kDies),
-                    static_cast<unsigned>(kTileTokens * a.num_topk + prefetch_ys),
-                    static_cast<unsigned>(rounds));
-    if (fat)
-      hipLaunchKernelGGL((ep_permute_tiles_kernel<true, 4>), grid, dim3(kPushThreads), 0, stream, a, tiles,
-                         prefetch_ys);
-    else
-      hipLaunchKernelGGL((ep_permute_tiles_kernel<true, 1>), grid, dim3(kPushThreads), 0, stream, a, tiles,
-                         prefetch_ys);
-    return hipGetLastError();
+    const int ys = kTileTokens * a.num_topk + prefetch_ys;
+    // Zeroed pads: extra rounds behind the copy, eight pad rows (one per die) per y.
+    const long long pad_rounds =
+        (pad_items > 0 && a.zero_pad_payload) ? (pad_items + static_cast<long long>(ys) * kDies - 1) / (static_cast<long long>(ys) * kDies) : 0;
+    if (rounds + pad_rounds > 65535 || parts * kDies > 65535) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(parts * kDies), static_cast<unsigned>(ys),
+                    static_cast<unsigned>(rounds + pad_rounds));
+    return fat ? launch_permute_tiles<4>(a, grid, tiles, rounds, stream)
+               : launch_permute_tiles<1>(a, grid, tiles, rounds, stream);
   }
   const int batches = (a.row_vecs + kWave - 1) / kWave;
-  const long long units = static_cast<long long>(a.num_tokens) * batches;
+  long long units = static_cast<long long>(a.num_tokens) * batches;
+  if (pad_items > 0) {
+    units += (pad_items + kWave - 1) / kWave;             // side data of the pad rows, one item per lane
+    if (a.zero_pad_payload) units += pad_items * batches;  // their payload, one unit per KiB
+  }
   const long long blocks = (units + kPushWaves - 1) / kPushWaves;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
   hipLaunchKernelGGL((ep_permute_kernel<1, true>), dim3(static_cast<unsigned>(blocks)), dim3(kPushThreads), 0,
@@ -545,14 +688,15 @@ hipError_t launch_permute_ranks(const RankPermuteArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_gather_rank_weights(const float* recv_topk_weights, const int* rank_row_map, int num_tokens,
-                                      int num_topk, int num_rows, float* combined_topk_weights,
+hipError_t launch_gather_rank_weights(const float* recv_topk_weights, const int64_t* recv_topk_idx,
+                                      const int* rank_row_map, int num_tokens, int num_topk, int num_rows,
+                                      float* combined_topk_weights, int64_t* combined_topk_idx,
                                       hipStream_t stream) {
   const long long total = static_cast<long long>(num_tokens) * num_topk;
   if (total == 0) return hipSuccess;
   hipLaunchKernelGGL(ep_gather_rank_weights_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
-                     stream, recv_topk_weights, rank_row_map, static_cast<int>(total), num_topk, num_rows,
-                     combined_topk_weights);
+                     stream, recv_topk_weights, recv_topk_idx, rank_row_map, static_cast<int>(total), num_topk,
+                     num_rows, combined_topk_weights, combined_topk_idx);
   return hipGetLastError();
 }
 
@@ -589,17 +733,6 @@ hipError_t launch_pull_indices(const int* recv_src_map, int num_rows, int tokens
   if (num_rows == 0) return hipSuccess;
   hipLaunchKernelGGL(ep_pull_indices_kernel, dim3((num_rows + 255) / 256), dim3(256), 0, stream, recv_src_map,
                      num_rows, tokens_per_source_rank, reinterpret_cast<int2*>(pull_indices));
-  return hipGetLastError();
-}
-
-hipError_t launch_pad_rows(const PermuteArgs& a, int expert_alignment, bool zero_payload, hipStream_t stream) {
-  // An expert has at most expert_alignment - 1 pad rows: one workgroup per possible pad row.
-  int per_expert = expert_alignment - 1;
-  if (per_expert < 1) return hipSuccess;
-  if (per_expert > 1024) per_expert = 1024;
-  if (!zero_payload) per_expert = 1;  // only the map entries: one workgroup per expert walks them
-  hipLaunchKernelGGL(ep_pad_rows_kernel, dim3(a.num_experts, per_expert), dim3(kPermuteThreads), 0, stream, a,
-                     zero_payload);
   return hipGetLastError();
 }
 

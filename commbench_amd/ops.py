@@ -14,7 +14,7 @@ split into `num_ranks` partitions:
         -> (recv_x, recv_topk_idx, recv_topk_weights, handle)            format: one row per token
     combine_ranks(y, handle, recv_topk_weights) -> combined_x[, weights]  and destination rank
     dispatch_cached / pull_indices                                        pull form from a source map
-    host_get_dispatch_layout / host_dispatch / host_combine               numpy in, numpy out
+    host_get_dispatch_layout / host_dispatch_layout / host_dispatch / host_combine    numpy in, numpy out
 
 torch is used for device memory and streams only; all arithmetic runs in the HIP kernels of
 libmi_ep.so.  Nothing here falls back to torch ops or to the CPU.
@@ -30,6 +30,9 @@ MAX_RANKS = 8
 MAX_TOPK = 8
 MAX_EXPERTS = 1024
 KEEP_PAD_PAYLOAD = 1   # MI_EP_DISPATCH_KEEP_PAD_PAYLOAD
+BY_TOKEN = 2           # MI_EP_DISPATCH_BY_TOKEN
+BY_DESTINATION = 4     # MI_EP_DISPATCH_BY_DESTINATION
+_SCHEDULE_FLAGS = {"auto": 0, "token": BY_TOKEN, "destination": BY_DESTINATION}
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -89,6 +92,8 @@ class DispatchHandle:
     slot_rel: torch.Tensor                 # int32[T, K]
     rank_slot_idx: Optional[torch.Tensor] = None   # int32[T, K], the prologue's dst_buffer_slot_idx
     route_order: Optional[torch.Tensor] = None     # int32[tiles * 256 * K, 4], routes in destination order
+    tile_rank_counts: Optional[torch.Tensor] = None  # int32[tiles, R], the prologue's rank_count_buffer
+    copied_topk_idx: Optional[torch.Tensor] = None   # int64[T, K], the kernel's own copy of topk_idx
     slot_map: Optional[torch.Tensor] = None        # int32[T, K]
     recv_src_map: Optional[torch.Tensor] = None    # int32[capacity]
     recv_topk_idx: Optional[torch.Tensor] = None   # int64[capacity]
@@ -123,6 +128,12 @@ class Buffer:
             _lib.check(lib.mi_ep_workspace_init(_ptr(self.workspace), nbytes, _stream()),
                        "mi_ep_workspace_init")
 
+    def set_wait_limit(self, max_polls: int) -> None:
+        """Bounds the device-side waits of later layout launches on this buffer (0 = default)."""
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.load().mi_ep_workspace_set_wait_limit(_ptr(self.workspace), max_polls, _stream()),
+                       "mi_ep_workspace_set_wait_limit")
+
     def status(self) -> None:
         """Raises if a device-side bounded wait ever expired on this workspace."""
         lib = _lib.load()
@@ -132,14 +143,19 @@ class Buffer:
 
     def dispatch_layout(self, topk_idx: torch.Tensor, expert_alignment: int = 1,
                         num_channels: int = 0, rank_slot_base: Optional[int] = None,
-                        route_order: bool = True) -> DispatchHandle:
+                        route_order: bool = True, tile_rank_counts: bool = False,
+                        copy_topk_idx: bool = False,
+                        cumulative_expert_stats: Optional[torch.Tensor] = None) -> DispatchHandle:
         """Fused single-pass layout: counts, flags, offsets, per-route segment positions, and
         (unless `route_order` is False) the per-tile destination order that lets dispatch write
         adjacent rows together.
 
         With `rank_slot_base` (the reference's scaleup_rank_idx * num_max_tokens_per_rank) the
         handle also carries `rank_slot_idx`, the deterministic prologue's per-rank slot table
-        (example078 .cu:36-40)."""
+        (example078 .cu:36-40); `tile_rank_counts` adds its per-tile rank counts (:34-35),
+        `copy_topk_idx` the kernel's own copy of the routing table (example080 .cu:33), and
+        `cumulative_expert_stats` (int32[E]) has this call's per-expert counts added to it
+        (example080 .cu:35,211-212)."""
         T, K = _check_routing(topk_idx, self.num_experts, self.num_ranks)
         _require(K == self.num_topk, "num_topk differs from the buffer's")
         _require(T <= self.num_max_tokens, "more tokens than the buffer was sized for")
@@ -162,11 +178,20 @@ class Buffer:
         if route_order and T > 0:
             h.route_order = torch.empty((lib.mi_ep_route_order_bytes(T, K) // 16, 4), dtype=torch.int32,
                                         device=dev)
+        if tile_rank_counts:
+            h.tile_rank_counts = torch.empty(((T + 255) // 256, R), dtype=torch.int32, device=dev)
+        if copy_topk_idx:
+            h.copied_topk_idx = torch.empty((T, K), dtype=torch.int64, device=dev)
+        if cumulative_expert_stats is not None:
+            _require(cumulative_expert_stats.is_cuda and cumulative_expert_stats.dtype == torch.int32
+                     and cumulative_expert_stats.is_contiguous() and cumulative_expert_stats.numel() == E,
+                     "cumulative_expert_stats must be a contiguous int32 [num_experts] GPU tensor")
         _lib.check(lib.mi_ep_dispatch_layout(
             _ptr(topk_idx), T, K, R, E, expert_alignment, num_channels,
             _ptr(h.num_tokens_per_rank), _ptr(h.num_tokens_per_expert), _ptr(h.is_token_in_rank),
             _ptr(h.expert_offsets), _ptr(h.psum_rank_rows), _ptr(h.channel_prefix_matrix),
             _ptr(h.slot_rel), _ptr(h.rank_slot_idx), rank_slot_base or 0, _ptr(h.route_order),
+            _ptr(h.tile_rank_counts), _ptr(h.copied_topk_idx), _ptr(cumulative_expert_stats),
             _ptr(self.workspace),
             self.workspace.numel(), _stream()), "mi_ep_dispatch_layout")
         return h
@@ -175,7 +200,7 @@ class Buffer:
                  topk_weights: Optional[torch.Tensor], expert_alignment: int = 1,
                  num_channels: int = 0, handle: Optional[DispatchHandle] = None,
                  capacity_rows: Optional[int] = None, rank_slot_base: Optional[int] = None,
-                 zero_pads: bool = True, column_major_recv_scales: bool = False):
+                 zero_pads: bool = True, column_major_recv_scales: bool = False, schedule: str = "auto"):
         """Layout (unless `handle` is given) + permute into the expert-contiguous buffer.
 
         Returns (recv_x, recv_scales, recv_src_map, handle).  Buffers hold `capacity_rows` rows
@@ -185,7 +210,10 @@ class Buffer:
         `scales` may be any 2-D float32 view (row- or column-major, padded); with
         `column_major_recv_scales` the returned recv_scales is a [capacity, S] view of a [S, capacity]
         allocation, the layout the reference's TMA-aligned scale tensors have.
+        `schedule` picks the copy kernel: "auto" (by shape and device), "token" or "destination";
+        the results are identical.
         """
+        _require(schedule in _SCHEDULE_FLAGS, 'schedule must be "auto", "token" or "destination"')
         if handle is None:
             handle = self.dispatch_layout(topk_idx, expert_alignment, num_channels, rank_slot_base)
         T, K, E = handle.num_tokens, handle.num_topk, handle.num_experts
@@ -223,7 +251,8 @@ class Buffer:
             _ptr(handle.expert_offsets), _ptr(handle.slot_rel), _ptr(handle.route_order),
             _ptr(handle.num_tokens_per_expert), T, K, E, handle.expert_alignment, row_bytes, num_scales,
             _ptr(recv_x), _ptr(recv_scales), rs_strides[0], rs_strides[1], _ptr(handle.recv_src_map),
-            _ptr(handle.recv_topk_idx), _ptr(handle.recv_topk_weights), _ptr(handle.slot_map), capacity_rows, 0 if zero_pads else KEEP_PAD_PAYLOAD, _stream()),
+            _ptr(handle.recv_topk_idx), _ptr(handle.recv_topk_weights), _ptr(handle.slot_map), capacity_rows,
+            (0 if zero_pads else KEEP_PAD_PAYLOAD) | _SCHEDULE_FLAGS[schedule], _stream()),
             "mi_ep_dispatch_strided_scales")
         return recv_x, recv_scales, handle.recv_src_map, handle
 
@@ -245,12 +274,15 @@ class RankDispatchHandle:
 
 def dispatch_ranks(buffer: "Buffer", x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Tensor,
                    topk_weights: Optional[torch.Tensor], num_max_tokens_per_rank: Optional[int] = None,
-                   rank_idx: int = 0, local_expert_ids: bool = False, expand: bool = False):
+                   rank_idx: int = 0, local_expert_ids: bool = False, expand: bool = False,
+                   column_major_recv_scales: bool = False):
     """The reference's dispatch in its own receive format: one row per (token, destination rank),
     ranks' rows in token order (deterministic mode).  Returns (recv_x, recv_topk_idx,
     recv_topk_weights, handle) as DeepEP's `buffer.dispatch` does (example080 bar.py:725);
     `rank_idx * num_max_tokens_per_rank` offsets the source token ids in the metadata.
-    With `expand`, the expert-contiguous dispatch runs too and the metadata names its rows."""
+    With `expand`, the expert-contiguous dispatch runs too and the metadata names its rows.
+    `scales` may be any 2-D float32 view; `column_major_recv_scales` returns them in a [S, rows]
+    allocation viewed as [rows, S] (the reference passes token and hidden strides, example081 .cu:31)."""
     T, K = _check_routing(topk_idx, buffer.num_experts, buffer.num_ranks)
     E, R, dev = buffer.num_experts, buffer.num_ranks, topk_idx.device
     max_tokens = T if num_max_tokens_per_rank is None else num_max_tokens_per_rank
@@ -265,12 +297,18 @@ def dispatch_ranks(buffer: "Buffer", x: torch.Tensor, scales: Optional[torch.Ten
     _require(row_bytes % 16 == 0, "row size must be a multiple of 16 bytes")
     S = 0
     if scales is not None:
-        _require(scales.dtype == torch.float32 and scales.dim() == 2 and scales.is_contiguous()
-                 and scales.shape[0] == T, "scales must be contiguous float32 [num_tokens, S]")
+        _require(scales.dtype == torch.float32 and scales.dim() == 2 and scales.shape[0] == T
+                 and min(scales.stride()) >= 0, "scales must be a float32 [num_tokens, S] tensor or view")
         S = scales.shape[1]
     cap = T * min(K, R)
     recv_x = torch.empty((cap, x.shape[1]), dtype=x.dtype, device=dev)
-    recv_scales = torch.empty((cap, S), dtype=torch.float32, device=dev) if scales is not None else None
+    recv_scales = None
+    if scales is not None and column_major_recv_scales:
+        recv_scales = torch.empty((S, cap), dtype=torch.float32, device=dev).t()
+    elif scales is not None:
+        recv_scales = torch.empty((cap, S), dtype=torch.float32, device=dev)
+    xs_strides = scales.stride() if scales is not None else (0, 0)
+    rs_strides = recv_scales.stride() if recv_scales is not None else (0, 0)
     recv_idx = torch.empty((cap, K), dtype=torch.int64, device=dev)
     recv_w = torch.empty((cap, K), dtype=torch.float32, device=dev)
     rh = RankDispatchHandle(
@@ -278,43 +316,58 @@ def dispatch_ranks(buffer: "Buffer", x: torch.Tensor, scales: Optional[torch.Ten
         recv_src_metadata=torch.empty((cap, 2 + K), dtype=torch.int32, device=dev),
         rank_row_map=torch.empty((T, K), dtype=torch.int32, device=dev),
         combine_map=torch.empty((T, K), dtype=torch.int32, device=dev), recv_scales=recv_scales)
-    _lib.check(_lib.load().mi_ep_dispatch_ranks(
-        _ptr(x), _ptr(scales), _ptr(topk_idx), _ptr(topk_weights), _ptr(h.rank_slot_idx), base,
-        _ptr(h.num_tokens_per_rank), _ptr(h.slot_map) if expand else None, T, K, R, E, row_bytes, S, base,
-        1 if local_expert_ids else 0, _ptr(recv_x), _ptr(recv_scales), _ptr(recv_idx), _ptr(recv_w),
-        _ptr(rh.recv_src_metadata), _ptr(rh.rank_row_map), _ptr(rh.combine_map), _ptr(rh.psum_rank_tokens),
-        cap, _stream()), "mi_ep_dispatch_ranks")
+    _lib.check(_lib.load().mi_ep_dispatch_ranks_strided_scales(
+        _ptr(x), _ptr(scales), xs_strides[0], xs_strides[1], _ptr(topk_idx), _ptr(topk_weights),
+        _ptr(h.rank_slot_idx), base, _ptr(h.num_tokens_per_rank), _ptr(h.slot_map) if expand else None, T, K, R,
+        E, row_bytes, S, base, 1 if local_expert_ids else 0, _ptr(recv_x), _ptr(recv_scales), rs_strides[0],
+        rs_strides[1], _ptr(recv_idx), _ptr(recv_w), _ptr(rh.recv_src_metadata), _ptr(rh.rank_row_map),
+        _ptr(rh.combine_map), _ptr(rh.psum_rank_tokens), cap, _stream()), "mi_ep_dispatch_ranks_strided_scales")
     return recv_x, recv_idx, recv_w, rh
 
 
 def combine_ranks(y: torch.Tensor, handle: RankDispatchHandle, recv_topk_weights: Optional[torch.Tensor] = None,
-                  bias=None):
+                  bias=None, recv_topk_idx: Optional[torch.Tensor] = None):
     """The reference's combine of the per-rank format: the ordered sum of the rows a token sent
     out, one per rank (+ biases); with `recv_topk_weights` also the weights that travelled
-    (combined_topk_weights, example082 bar.py:757-765)."""
+    (combined_topk_weights, example082 bar.py:757-765), with `recv_topk_idx` also the expert ids
+    (combined_topk_idx, example083 .cu:26).  Returns combined_x, then the weights, then the ids,
+    as far as they were asked for."""
     out = combine(y, handle.combine_map, None, bias)
-    if recv_topk_weights is None:
+    if recv_topk_weights is None and recv_topk_idx is None:
         return out
     T, K = handle.rank_row_map.shape
-    _require(recv_topk_weights.dtype == torch.float32 and recv_topk_weights.is_contiguous()
-             and recv_topk_weights.dim() == 2 and recv_topk_weights.shape[1] == K,
-             "recv_topk_weights must be contiguous float32 [rows, num_topk]")
-    out_w = torch.empty((T, K), dtype=torch.float32, device=y.device)
+    rows = None
+    out_w = out_i = None
+    if recv_topk_weights is not None:
+        _require(recv_topk_weights.dtype == torch.float32 and recv_topk_weights.is_contiguous()
+                 and recv_topk_weights.dim() == 2 and recv_topk_weights.shape[1] == K,
+                 "recv_topk_weights must be contiguous float32 [rows, num_topk]")
+        rows = recv_topk_weights.shape[0]
+        out_w = torch.empty((T, K), dtype=torch.float32, device=y.device)
+    if recv_topk_idx is not None:
+        _require(recv_topk_idx.dtype == torch.int64 and recv_topk_idx.is_contiguous()
+                 and recv_topk_idx.dim() == 2 and recv_topk_idx.shape[1] == K
+                 and (rows is None or recv_topk_idx.shape[0] == rows),
+                 "recv_topk_idx must be contiguous int64 [rows, num_topk]")
+        rows = recv_topk_idx.shape[0]
+        out_i = torch.empty((T, K), dtype=torch.int64, device=y.device)
     _lib.check(_lib.load().mi_ep_combine_rank_weights(
-        _ptr(recv_topk_weights), _ptr(handle.rank_row_map), T, K, recv_topk_weights.shape[0], _ptr(out_w),
-        _stream()), "mi_ep_combine_rank_weights")
-    return out, out_w
+        _ptr(recv_topk_weights), _ptr(recv_topk_idx), _ptr(handle.rank_row_map), T, K, rows, _ptr(out_w),
+        _ptr(out_i), _stream()), "mi_ep_combine_rank_weights")
+    return tuple(t for t in (out, out_w, out_i) if t is not None)
 
 
 def combine(y: torch.Tensor, slot_map: Union[torch.Tensor, DispatchHandle],
             topk_weights: Optional[torch.Tensor] = None,
             bias: Union[None, torch.Tensor, Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]] = None,
-            recv_topk_weights: Optional[torch.Tensor] = None):
+            recv_topk_weights: Optional[torch.Tensor] = None,
+            recv_topk_idx: Optional[torch.Tensor] = None):
     """combined_x[t] = bf16(sum_k w[t,k] * y[slot_map[t,k]] (+ biases)), fp32 accumulation.
 
     topk_weights=None gives the reference's plain ordered sum.  When `recv_topk_weights` (the
     per-row weights that travelled with dispatch) is given, also returns them gathered back to
-    [num_tokens, num_topk], as the reference's combined_topk_weights.
+    [num_tokens, num_topk], as the reference's combined_topk_weights; `recv_topk_idx` (the per-row
+    expert ids) likewise comes back as combined_topk_idx, after the weights.
     """
     if isinstance(slot_map, DispatchHandle):
         _require(slot_map.slot_map is not None, "handle has not been through dispatch")
@@ -344,13 +397,18 @@ def combine(y: torch.Tensor, slot_map: Union[torch.Tensor, DispatchHandle],
     out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
     out_w = (torch.empty((T, K), dtype=torch.float32, device=dev)
              if recv_topk_weights is not None else None)
+    out_i = (torch.empty((T, K), dtype=torch.int64, device=dev)
+             if recv_topk_idx is not None else None)
+    if recv_topk_idx is not None:
+        _require(recv_topk_idx.dtype == torch.int64 and recv_topk_idx.is_contiguous(),
+                 "recv_topk_idx must be contiguous int64 [rows]")
     lib = _lib.load()
     _lib.check(lib.mi_ep_combine(_ptr(y), y.shape[0], _ptr(slot_map), _ptr(topk_weights), _ptr(bias_0),
-                                 _ptr(bias_1), _ptr(recv_topk_weights), T, K, H, _ptr(out),
-                                 _ptr(out_w), _stream()), "mi_ep_combine")
-    if out_w is not None:
-        return out, out_w
-    return out
+                                 _ptr(bias_1), _ptr(recv_topk_weights), _ptr(recv_topk_idx), T, K, H,
+                                 _ptr(out), _ptr(out_w), _ptr(out_i), _stream()), "mi_ep_combine")
+    if out_w is None and out_i is None:
+        return out
+    return tuple(t for t in (out, out_w, out_i) if t is not None)
 
 
 def dispatch(x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Tensor,
@@ -412,6 +470,26 @@ def pull_indices(recv_src_map: torch.Tensor, tokens_per_source_rank: int,
     return out
 
 
+def device_traits() -> dict:
+    """What the runtime reports for the current device: compute units, accelerator dies, L2 bytes
+    per die (the destination-order copy is tuned for 8 dies with 4 MiB each)."""
+    import ctypes
+    cus, dies, l2 = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    _lib.check(_lib.load().mi_ep_device_traits(ctypes.byref(cus), ctypes.byref(dies), ctypes.byref(l2), _stream()),
+               "mi_ep_device_traits")
+    return {"compute_units": cus.value, "dies": dies.value, "l2_bytes": l2.value}
+
+
+def dispatch_schedule_for(num_tokens: int, num_topk: int, num_experts: int, row_bytes: int) -> str:
+    """The copy kernel `schedule="auto"` picks for a shape on the current device."""
+    traits = device_traits()
+    code = _lib.load().mi_ep_dispatch_schedule_for(num_tokens, num_topk, num_experts, row_bytes,
+                                                   traits["dies"], traits["l2_bytes"])
+    if code not in (BY_TOKEN, BY_DESTINATION):
+        _lib.check(code if code != 0 else -22, "mi_ep_dispatch_schedule_for")
+    return "destination" if code == BY_DESTINATION else "token"
+
+
 def copy_yardstick(dst: torch.Tensor, src: torch.Tensor) -> None:
     """16-byte streaming copy of src into dst (same byte size), the measured-bandwidth yardstick."""
     nbytes = src.numel() * src.element_size()
@@ -449,6 +527,38 @@ def host_get_dispatch_layout(topk_idx, num_experts: int, num_ranks: int):
         _np_ptr(topk_idx), _np_ptr(per_rank), None, _np_ptr(per_expert), _np_ptr(flags), T, K, num_ranks,
         num_experts), "mi_ep_host_get_dispatch_layout")
     return per_rank, per_expert, flags
+
+
+def host_dispatch_layout(topk_idx, num_experts: int, num_ranks: int, expert_alignment: int = 1,
+                         num_channels: int = 0, rank_slot_base: int = 0, cumulative_expert_stats=None):
+    """The fused layout on host arrays: a dict with every output of mi_ep_dispatch_layout
+    (`cumulative_expert_stats`, int32[E], is updated in place when given)."""
+    import numpy as np
+    topk_idx = _np(topk_idx, np.int64)
+    _require(topk_idx.ndim == 2, "topk_idx must be [num_tokens, num_topk]")
+    T, K = topk_idx.shape
+    E, R = num_experts, num_ranks
+    if cumulative_expert_stats is not None:
+        _require(cumulative_expert_stats.dtype == np.int32 and cumulative_expert_stats.flags.c_contiguous
+                 and cumulative_expert_stats.shape == (E,), "cumulative_expert_stats must be int32 [num_experts]")
+    order_rows = _lib.load().mi_ep_route_order_bytes(T, K) // 16
+    out = dict(
+        num_tokens_per_rank=np.empty(R, dtype=np.int32), num_tokens_per_expert=np.empty(E, dtype=np.int32),
+        is_token_in_rank=np.empty((T, R), dtype=np.bool_), expert_offsets=np.empty(E + 1, dtype=np.int32),
+        psum_rank_rows=np.empty(R, dtype=np.int32),
+        channel_prefix_matrix=np.empty((R, num_channels), dtype=np.int32) if num_channels > 0 else None,
+        slot_rel=np.empty((T, K), dtype=np.int32), rank_slot_idx=np.empty((T, K), dtype=np.int32),
+        route_order=np.empty((order_rows, 4), dtype=np.int32),
+        tile_rank_counts=np.empty(((T + 255) // 256, R), dtype=np.int32),
+        copied_topk_idx=np.empty((T, K), dtype=np.int64))
+    _lib.check(_lib.load().mi_ep_host_dispatch_layout(
+        _np_ptr(topk_idx), T, K, R, E, expert_alignment, num_channels, _np_ptr(out["num_tokens_per_rank"]),
+        _np_ptr(out["num_tokens_per_expert"]), _np_ptr(out["is_token_in_rank"]), _np_ptr(out["expert_offsets"]),
+        _np_ptr(out["psum_rank_rows"]), _np_ptr(out["channel_prefix_matrix"]), _np_ptr(out["slot_rel"]),
+        _np_ptr(out["rank_slot_idx"]), rank_slot_base, _np_ptr(out["route_order"]),
+        _np_ptr(out["tile_rank_counts"]), _np_ptr(out["copied_topk_idx"]), _np_ptr(cumulative_expert_stats)),
+        "mi_ep_host_dispatch_layout")
+    return out
 
 
 def host_dispatch(x, scales, topk_idx, topk_weights, num_experts: int, num_ranks: int,

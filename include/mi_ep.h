@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define MI_EP_ABI_VERSION 1
+#define MI_EP_ABI_VERSION 2
 
 #define MI_EP_OK 0
 #define MI_EP_EINVAL (-22)    /* argument out of range or NULL where required */
@@ -31,7 +31,6 @@ extern "C" {
 
 /* Limits.  Ranks and top-k follow the reference's constructor checks
  * (example042_deepep_dispatch_layout/nv/empty_deepep_dispatch_layout.cu:43,46,96-107). */
-#define MI_EP_DISPATCH_KEEP_PAD_PAYLOAD 1
 #define MI_EP_MAX_RANKS 8
 #define MI_EP_MAX_TOPK 8
 #define MI_EP_MAX_EXPERTS 1024
@@ -68,21 +67,28 @@ int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
  * workspace gave up a bounded device-side wait since the last init. */
 int mi_ep_workspace_status(const void* workspace, void* stream);
 
-/* Test hook, process-wide: bounds the number of unsuccessful polls of one device-side wait in
- * later mi_ep_dispatch_layout launches: a wait gives up at its max_polls-th unsuccessful poll in
- * a row (0 restores the default of about four million).  A launch
- * whose wait expires still terminates; its outputs are then unspecified and the workspace
- * reports MI_EP_ETIMEDOUT until it is initialised again.  The reference's counterpart is the
- * kNumTimeoutCycles template argument of dispatch_impl
- * (example080_deepep_jit_dispatch_payload/nv/empty_deepep_jit_dispatch_payload.cu:29,122-143). */
-int mi_ep_set_wait_limit(unsigned int max_polls);
-/* Test and measurement hook, process-wide: which copy kernel later mi_ep_dispatch calls use.
- * 0 = chosen by shape (default), 1 = by token (wave per token and KiB, rows scattered),
- * 2 = by destination whenever route_order is given.  Results are identical. */
-int mi_ep_set_dispatch_schedule(int schedule);
-/* The kernel the default picks for a shape when route_order is given: 1 or 2 as above
- * (kernel symbols ep_permute_kernel and ep_permute_tiles_kernel), or MI_EP_EINVAL. */
-int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, int row_bytes);
+/* Bounds the device-side waits of later mi_ep_dispatch_layout launches on THIS workspace: a wait
+ * gives up at its max_polls-th unsuccessful poll in a row (0 restores the default of about four
+ * million, a few seconds).  Enqueue-only; mi_ep_workspace_init resets it to the default.  A launch
+ * whose wait expires still terminates; its outputs are then unspecified, dispatch calls fed with
+ * them write no row outside the destination buffer, and the workspace reports MI_EP_ETIMEDOUT until
+ * it is initialised again: check mi_ep_workspace_status before trusting the outputs of a launch that
+ * may have timed out.  The reference's counterpart is the kNumTimeoutCycles template argument of
+ * dispatch_impl (example080_deepep_jit_dispatch_payload/nv/empty_deepep_jit_dispatch_payload.cu:29,122-143). */
+int mi_ep_workspace_set_wait_limit(void* workspace, unsigned int max_polls, void* stream);
+
+/* What the destination-order copy kernel assumes of a device, as the runtime reports it for the
+ * device `stream` belongs to (the current device for NULL): compute units, accelerator dies
+ * (XCCs) and bytes of L2 per die; any pointer may be NULL.  The kernel is tuned for 8 dies that
+ * take workgroups round-robin and 4 MiB of L2 each; on anything else (another partition mode,
+ * another part) mi_ep_dispatch takes the token-order kernel unless told otherwise. */
+int mi_ep_device_traits(int* compute_units, int* dies, int* l2_bytes, void* stream);
+/* The kernel mi_ep_dispatch picks by itself for a shape when route_order is given, on a device
+ * with these traits (from mi_ep_device_traits): MI_EP_DISPATCH_BY_TOKEN or
+ * MI_EP_DISPATCH_BY_DESTINATION (kernel symbols ep_permute_kernel and ep_permute_tiles_kernel), or
+ * MI_EP_EINVAL.  Touches no device. */
+int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, int row_bytes, int dies,
+                                int l2_bytes);
 
 /*
  * Fused single-pass layout: everything the reference spreads over
@@ -91,7 +97,7 @@ int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, i
  *   example078 (deterministic slots, empty_deepep_jit_dispatch_deterministic_prologue.cu:27-43),
  *   example080 notify role (histogram, aligned exclusive expert psum, inclusive rank
  *   psum, empty_deepep_jit_dispatch_payload.cu:78-107,197-239).
- * Outputs (any of the last five may be NULL):
+ * Outputs:
  *   num_tokens_per_rank / num_tokens_per_expert / is_token_in_rank   as above
  *   expert_offsets      int32[num_experts + 1]; off[0] = 0,
  *                       off[e+1] = off[e] + round_up(count[e], expert_alignment)
@@ -114,13 +120,23 @@ int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, i
  *                       recv_x in destination order (no counterpart in the reference, whose
  *                       senders push token by token; the nearest relative is the sorted pull
  *                       list of example056 compute_dispatch_indices, :521-564).  16-byte aligned.
+ *   tile_rank_counts    int32[ceil(num_tokens / 256), num_ranks]; tokens of each 256-token tile
+ *                       flagged for each rank: the one-GPU form of rank_count_buffer[sm, rank]
+ *                       (example078 .cu:20,34-35), a tile standing for an SM's share of the tokens
+ *   copied_topk_idx     int64[num_tokens, num_topk]; verbatim copy of topk_idx for the handle to
+ *                       keep (example080 .cu:33)
+ *   cumulative_expert_stats  int32[num_experts], NOT overwritten: every launch adds its
+ *                       num_tokens_per_expert (unaligned counts) to it
+ *                       (cumulative_local_expert_recv_stats, example080 .cu:35,211-212)
+ * Any of the outputs from expert_offsets on may be NULL.
  */
 int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
                           int num_experts, int expert_alignment, int num_channels,
                           int* num_tokens_per_rank, int* num_tokens_per_expert,
                           bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
                           int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
-                          int rank_slot_base, int* route_order, void* workspace,
+                          int rank_slot_base, int* route_order, int* tile_rank_counts,
+                          int64_t* copied_topk_idx, int* cumulative_expert_stats, void* workspace,
                           size_t workspace_bytes, void* stream);
 /*
  * mi_ep_dispatch_layout without a workspace argument and without any allocation.  It has no
@@ -147,7 +163,9 @@ int mi_ep_dispatch_layout_static(const int64_t* topk_idx, int num_tokens, int nu
                                  int* num_tokens_per_rank, int* num_tokens_per_expert,
                                  bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
                                  int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
-                                 int rank_slot_base, int* route_order, int* timeout_report, void* stream);
+                                 int rank_slot_base, int* route_order, int* tile_rank_counts,
+                                 int64_t* copied_topk_idx, int* cumulative_expert_stats,
+                                 int* timeout_report, void* stream);
 /* Bytes of route_order for this shape. */
 size_t mi_ep_route_order_bytes(int num_tokens, int num_topk);
 
@@ -169,17 +187,26 @@ size_t mi_ep_route_order_bytes(int num_tokens, int num_topk);
  *   recv_topk_weights float[capacity_rows] or NULL: gate weight of the row's route; 0 pad
  *   slot_map     int32[num_tokens, num_topk]: absolute row of each route, -1 non-routes
  * Rows >= capacity_rows are never written.  With expert_alignment > 1 pad rows are
- * zero-filled; num_tokens_per_expert (from the layout call) locates them and may be
- * NULL when expert_alignment == 1.  flags: 0, or MI_EP_DISPATCH_KEEP_PAD_PAYLOAD to leave the
- * payload and scales of pad rows untouched (their map entries are still written: source -1,
- * expert -1, weight 0), for consumers that never look at what a pad row produces -- at
- * alignment 128 the zero fill is a fifth of the copy.
+ * zero-filled by further workgroups of the same launch; num_tokens_per_expert (from the layout
+ * call) locates them and may be NULL when expert_alignment == 1.
+ *   flags        0, or an OR of
+ *                MI_EP_DISPATCH_KEEP_PAD_PAYLOAD  leave the payload and scales of pad rows untouched,
+ *                  as the reference's receive buffer is (its harness pads to 128 rows and only reads
+ *                  the received ones, example080 build_and_run.py:718,728-748); their map entries are
+ *                  still written (source -1, expert -1, weight 0).  At alignment 128 the zero fill is
+ *                  a fifth of the copy's bytes.
+ *                MI_EP_DISPATCH_BY_TOKEN / MI_EP_DISPATCH_BY_DESTINATION  (at most one) the copy
+ *                  kernel to use instead of the one chosen by shape and device; by destination needs
+ *                  route_order.  Results are identical.
  *   route_order  the layout call's table for the same topk_idx, or NULL.  The outputs are the
  *                same either way; with it, large shapes are copied in destination order
  *                (adjacent rows of recv_x written together, sources re-read from the L2 of the
  *                die that owns the tile), which the HBM write path takes ~14 % faster than
  *                rows scattered token by token.
  */
+#define MI_EP_DISPATCH_KEEP_PAD_PAYLOAD 1
+#define MI_EP_DISPATCH_BY_TOKEN 2
+#define MI_EP_DISPATCH_BY_DESTINATION 4
 int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
                    const float* topk_weights, const int* expert_offsets, const int* slot_rel,
                    const int* route_order, const int* num_tokens_per_expert, int num_tokens, int num_topk,
@@ -235,9 +262,15 @@ int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long lon
  *                     mi_ep_combine(y, rows, combine_map, topk_weights = NULL, ...) is then the
  *                     reference's combine of this format (an ordered sum of the ranks' rows)
  * Rows at or beyond capacity_rows are dropped; min(num_topk, num_ranks) * num_tokens always fit.
- * mi_ep_combine_rank_weights returns the weights that travelled with the rows:
- * [t,k] = recv_topk_weights[rank_row_map[t,k], k], 0 for non-routes (combined_topk_weights,
- * example082 build_and_run.py:765).
+ * mi_ep_dispatch_ranks_strided_scales is the same call with the scale factors addressed through
+ * (token, hidden) strides in 4-byte elements on both sides, as the reference's epilogue takes them
+ * (recv_sf_token_stride, recv_sf_hidden_stride, example081 .cu:31); mi_ep_dispatch_ranks is that
+ * call with strides (num_scales, 1).
+ * mi_ep_combine_rank_weights returns what travelled with the rows, gathered back per route:
+ * combined_topk_weights[t,k] = recv_topk_weights[rank_row_map[t,k], k] (0 for non-routes;
+ * example082 build_and_run.py:765) and combined_topk_idx[t,k] = recv_topk_idx[rank_row_map[t,k], k]
+ * as stored (-1 for non-routes; combined_topk_idx of the reduce epilogue, example083 .cu:26).
+ * Either pair of pointers may be NULL, not both.
  */
 int mi_ep_dispatch_ranks(const void* x, const float* x_scales, const int64_t* topk_idx,
                          const float* topk_weights, const int* rank_slot_idx, int rank_slot_base,
@@ -247,8 +280,20 @@ int mi_ep_dispatch_ranks(const void* x, const float* x_scales, const int64_t* to
                          int64_t* recv_topk_idx, float* recv_topk_weights, int* recv_src_metadata,
                          int* rank_row_map, int* combine_map, int* psum_rank_tokens, int capacity_rows,
                          void* stream);
-int mi_ep_combine_rank_weights(const float* recv_topk_weights, const int* rank_row_map, int num_tokens,
-                               int num_topk, int num_rows, float* combined_topk_weights, void* stream);
+int mi_ep_dispatch_ranks_strided_scales(const void* x, const float* x_scales, long long x_scales_token_stride,
+                                        long long x_scales_hidden_stride, const int64_t* topk_idx,
+                                        const float* topk_weights, const int* rank_slot_idx, int rank_slot_base,
+                                        const int* num_tokens_per_rank, const int* expand_slot_map,
+                                        int num_tokens, int num_topk, int num_ranks, int num_experts,
+                                        int row_bytes, int num_scales, int source_token_base,
+                                        int local_expert_ids, void* recv_x, float* recv_scales,
+                                        long long recv_scales_token_stride, long long recv_scales_hidden_stride,
+                                        int64_t* recv_topk_idx, float* recv_topk_weights,
+                                        int* recv_src_metadata, int* rank_row_map, int* combine_map,
+                                        int* psum_rank_tokens, int capacity_rows, void* stream);
+int mi_ep_combine_rank_weights(const float* recv_topk_weights, const int64_t* recv_topk_idx,
+                               const int* rank_row_map, int num_tokens, int num_topk, int num_rows,
+                               float* combined_topk_weights, int64_t* combined_topk_idx, void* stream);
 
 /*
  * Pull-mode dispatch with a map from an earlier dispatch (the reference's cached mode,
@@ -293,11 +338,15 @@ int mi_ep_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_sou
  *   recv_topk_weights / combined_topk_weights   both NULL, or float[rows] in and
  *                float[num_tokens, num_topk] out: the weights that travelled with the
  *                rows, gathered back per route (0 for non-routes)
+ *   recv_topk_idx / combined_topk_idx   both NULL, or int64[rows] in and
+ *                int64[num_tokens, num_topk] out: the expert ids that travelled with the rows
+ *                (-1 for non-routes; combined_topk_idx, example083 .cu:26)
  */
 int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
                   const void* bias_0, const void* bias_1, const float* recv_topk_weights,
-                  int num_tokens, int num_topk, int hidden, void* combined_x,
-                  float* combined_topk_weights, void* stream);
+                  const int64_t* recv_topk_idx, int num_tokens, int num_topk, int hidden,
+                  void* combined_x, float* combined_topk_weights, int64_t* combined_topk_idx,
+                  void* stream);
 
 /*
  * Host-pointer twins: the same operations with every pointer in ordinary host memory.  Each call
@@ -306,6 +355,10 @@ int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float*
  * device-side pipeline (the reference's harnesses keep their data in host vectors between
  * hipMemcpy calls, example042 .cu:243-293); transfers dominate their time.
  *   mi_ep_host_get_dispatch_layout  twin of mi_ep_get_dispatch_layout
+ *   mi_ep_host_dispatch_layout      twin of mi_ep_dispatch_layout: same arguments and outputs without
+ *                                   the workspace; cumulative_expert_stats is read and written
+ *                                   (the running totals continue from the caller's values);
+ *                                   route_order entries past the last token come back as zeros
  *   mi_ep_host_dispatch             layout + dispatch in one call: the layout outputs
  *                                   (num_tokens_per_rank / _expert, is_token_in_rank, any of them
  *                                   may be NULL) and expert_offsets come back with the permuted
@@ -317,6 +370,12 @@ int mi_ep_host_get_dispatch_layout(const int64_t* topk_idx, int* num_tokens_per_
                                    int* num_tokens_per_rdma_rank, int* num_tokens_per_expert,
                                    bool* is_token_in_rank, int num_tokens, int num_topk, int num_ranks,
                                    int num_experts);
+int mi_ep_host_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
+                               int num_experts, int expert_alignment, int num_channels,
+                               int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
+                               int* expert_offsets, int* psum_rank_rows, int* channel_prefix_matrix,
+                               int* slot_rel, int* rank_slot_idx, int rank_slot_base, int* route_order,
+                               int* tile_rank_counts, int64_t* copied_topk_idx, int* cumulative_expert_stats);
 int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
                         const float* topk_weights, int num_tokens, int num_topk, int num_ranks,
                         int num_experts, int expert_alignment, int row_bytes, int num_scales,

@@ -95,6 +95,8 @@ struct DispatchHandle {
   int* slot_rel = nullptr;               // [T, K]
   int* rank_slot_idx = nullptr;          // [T, K] the deterministic prologue's table (base 0)
   int* route_order = nullptr;            // [tiles * 256 * K, 4] routes in destination order
+  int* tile_rank_counts = nullptr;       // [tiles, R] the prologue's rank_count_buffer, a tile per SM share
+  int64_t* copied_topk_idx = nullptr;    // [T, K] the layout kernel's own copy of topk_idx
   int* slot_map = nullptr;               // [T, K]
   int* recv_src_map = nullptr;           // [capacity]
   int64_t* recv_topk_idx = nullptr;      // [capacity]
@@ -136,6 +138,8 @@ class ExpertParallelBuffer {
     MI_EP_HIP_CHECK(hipMalloc(&h_.rank_combine_map, sizeof(int) * (tk + 1)));
     MI_EP_HIP_CHECK(hipMalloc(&h_.psum_rank_tokens, sizeof(int) * num_ranks));
     MI_EP_HIP_CHECK(hipMalloc(&h_.route_order, mi_ep_route_order_bytes(num_max_tokens, num_topk) + 16));
+    MI_EP_HIP_CHECK(hipMalloc(&h_.tile_rank_counts, sizeof(int) * ((num_max_tokens + 255) / 256 + 1) * num_ranks));
+    MI_EP_HIP_CHECK(hipMalloc(&h_.copied_topk_idx, sizeof(int64_t) * (tk + 1)));
     MI_EP_HIP_CHECK(hipMalloc(&h_.slot_map, sizeof(int) * (tk + 1)));
     MI_EP_HIP_CHECK(hipMalloc(&h_.recv_src_map, sizeof(int) * (capacity_ + 1)));
     MI_EP_HIP_CHECK(hipMalloc(&h_.recv_topk_idx, sizeof(int64_t) * (capacity_ + 1)));
@@ -148,7 +152,8 @@ class ExpertParallelBuffer {
     void* owned[] = {workspace_, h_.num_tokens_per_rank, h_.num_tokens_per_expert, h_.is_token_in_rank,
                      h_.expert_offsets, h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel,
                      h_.rank_slot_idx, h_.rank_row_map, h_.rank_combine_map, h_.psum_rank_tokens,
-                     h_.route_order, h_.slot_map, h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights};
+                     h_.route_order, h_.slot_map, h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights,
+                     h_.tile_rank_counts, h_.copied_topk_idx};
     for (void* p : owned)
       if (p != nullptr) (void)hipFree(p);
   }
@@ -158,6 +163,9 @@ class ExpertParallelBuffer {
 
   int capacity_rows() const { return capacity_; }
   const DispatchHandle& handle() const { return h_; }
+  // Running per-expert totals (int32[E], device memory of the caller): every later layout call adds
+  // its counts (the reference's cumulative_local_expert_recv_stats); nullptr switches it off.
+  void set_cumulative_expert_stats(int* d_stats) { cumulative_expert_stats_ = d_stats; }
 
   // Fused layout: counts, flags, offsets, per-route segment positions (and channel prefixes).
   // with_rank_slots also fills rank_slot_idx, the deterministic prologue's per-rank slot table.
@@ -170,20 +178,23 @@ class ExpertParallelBuffer {
                                       h_.num_tokens_per_expert, h_.is_token_in_rank, h_.expert_offsets,
                                       h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel,
                                       with_rank_slots ? h_.rank_slot_idx : nullptr, /*rank_slot_base=*/0, h_.route_order,
+                                      h_.tile_rank_counts, h_.copied_topk_idx, cumulative_expert_stats_,
                                       workspace_, workspace_bytes_, stream));
     return h_;
   }
 
   // Layout + permute.  recv_x / recv_scales hold capacity_rows() rows; scales may be null.
+  // flags: MI_EP_DISPATCH_* (pad payload kept, copy kernel forced).
   const DispatchHandle& dispatch(const void* d_x, const float* d_scales, const TopkIdx* d_topk_idx,
                                  const float* d_topk_weights, int num_tokens, int row_bytes, int num_scales,
-                                 void* d_recv_x, float* d_recv_scales, hipStream_t stream = 0) {
+                                 void* d_recv_x, float* d_recv_scales, hipStream_t stream = 0,
+                                 int flags = 0) {
     get_dispatch_layout(d_topk_idx, num_tokens, stream);
     MI_EP_CHECK(mi_ep_dispatch(d_x, d_scales, d_topk_idx, d_topk_weights, h_.expert_offsets, h_.slot_rel,
                                h_.route_order, h_.num_tokens_per_expert, num_tokens, num_topk_, num_experts_,
                                h_.expert_alignment, row_bytes, num_scales, d_recv_x, d_recv_scales,
                                h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights, h_.slot_map,
-                               capacity_, /*flags=*/0, stream));
+                               capacity_, flags, stream));
     return h_;
   }
 
@@ -210,18 +221,22 @@ class ExpertParallelBuffer {
   // The reference's combine of that format: the ordered sum of the rows a token sent out (+ biases).
   void combine_ranks(const void* d_y, int num_rows, const void* d_bias_0, const void* d_bias_1, int hidden,
                      void* d_combined_x, hipStream_t stream = 0) const {
-    MI_EP_CHECK(mi_ep_combine(d_y, num_rows, h_.rank_combine_map, nullptr, d_bias_0, d_bias_1, nullptr,
-                              h_.num_tokens, num_topk_, hidden, d_combined_x, nullptr, stream));
+    MI_EP_CHECK(mi_ep_combine(d_y, num_rows, h_.rank_combine_map, nullptr, d_bias_0, d_bias_1, nullptr, nullptr,
+                              h_.num_tokens, num_topk_, hidden, d_combined_x, nullptr, nullptr, stream));
   }
 
   // combined_x[t] = bf16(sum_k w[t,k] * y[slot_map[t,k]] + bias_0 + bias_1); null weights = plain sum.
   // d_y holds num_rows rows (capacity_rows() when it is the buffer dispatch filled).
+  // d_combined_topk_weights / d_combined_topk_idx (optional) receive the weights / expert ids that
+  // travelled with the rows.
   void combine(const void* d_y, int num_rows, const float* d_topk_weights, const void* d_bias_0,
                const void* d_bias_1, int hidden, void* d_combined_x,
-               float* d_combined_topk_weights = nullptr, hipStream_t stream = 0) const {
+               float* d_combined_topk_weights = nullptr, hipStream_t stream = 0,
+               int64_t* d_combined_topk_idx = nullptr) const {
     MI_EP_CHECK(mi_ep_combine(d_y, num_rows, h_.slot_map, d_topk_weights, d_bias_0, d_bias_1,
                               d_combined_topk_weights != nullptr ? h_.recv_topk_weights : nullptr,
-                              h_.num_tokens, num_topk_, hidden, d_combined_x, d_combined_topk_weights,
+                              d_combined_topk_idx != nullptr ? h_.recv_topk_idx : nullptr, h_.num_tokens,
+                              num_topk_, hidden, d_combined_x, d_combined_topk_weights, d_combined_topk_idx,
                               stream));
   }
 
@@ -240,6 +255,7 @@ class ExpertParallelBuffer {
   int capacity_ = 0;
   void* workspace_ = nullptr;
   size_t workspace_bytes_ = 0;
+  int* cumulative_expert_stats_ = nullptr;
   DispatchHandle h_;
 };
 

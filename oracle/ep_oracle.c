@@ -36,6 +36,13 @@
  *   ep_oracle_combine           example083_deepep_jit_combine_reduce_epilogue/nv/
  *                               empty_deepep_jit_combine_reduce_epilogue.cu:23-53
  *                               (fp32 accumulate over up to K rows, two biases, bf16 out)
+ *   ep_oracle_gather_weights,
+ *   ep_oracle_gather_idx        the same epilogue's combined_topk_weights / combined_topk_idx (:25-26):
+ *                               what travelled with each route's row, read back per (token, slot);
+ *                               ep_oracle_gather_rank_side the same for the per-rank format's [rows, K] tables
+ *   ep_oracle_tile_rank_counts  example078 .cu:20,34-35 (rank_count_buffer[sm, rank]) with a block of
+ *                               consecutive tokens standing for an SM's share
+ *   ep_oracle_accumulate_stats  example080 .cu:35,211-212 (cumulative_local_expert_recv_stats += counts)
  *
  * Pinning (what checks this file, beyond the kernels agreeing with it):
  *   layout           the reference's 13 closed-form correctness cases with
@@ -53,6 +60,9 @@
  *   pull indices     the closed form of the ThunderKittens example's own generator
  *   combine          exact rational arithmetic rounded once per fma (python ints),
  *                    integer-valued exact sums, K=1 copy, closed forms
+ *   gather idx / rank side   numpy fancy indexing with a mask
+ *   tile rank counts numpy add.reduceat over the flag matrix; column sums == per-rank counts
+ *   accumulate stats numpy += over several calls
  *   bf16 codec       exhaustive against torch.bfloat16 (fixtures in tests/golden)
  * Parity unpinned: the order in which two bias rows are added in the reference's
  * combine epilogue (its arithmetic lives in the un-vendored DeepEP tree); this
@@ -496,6 +506,45 @@ void ep_oracle_gather_weights(const float* recv_topk_weights, const int* slot_ma
                               int num_topk, float* combined_topk_weights) {
   for (size_t i = 0; i < (size_t)num_tokens * num_topk; ++i)
     combined_topk_weights[i] = slot_map[i] >= 0 ? recv_topk_weights[slot_map[i]] : 0.0f;
+}
+
+/* combined_topk_idx[t,k] = recv_topk_idx[slot_map[t,k]], -1 for non-routes. */
+void ep_oracle_gather_idx(const int64_t* recv_topk_idx, const int* slot_map, int num_tokens, int num_topk,
+                          int64_t* combined_topk_idx) {
+  for (size_t i = 0; i < (size_t)num_tokens * num_topk; ++i)
+    combined_topk_idx[i] = slot_map[i] >= 0 ? recv_topk_idx[slot_map[i]] : -1;
+}
+
+/* The per-rank format keeps K weights and K ids per row: route (t,k) reads column k of the row
+ * that carries it (rank_row_map[t,k]); 0 / -1 for non-routes.  Either output may be NULL. */
+void ep_oracle_gather_rank_side(const float* recv_topk_weights, const int64_t* recv_topk_idx,
+                                const int* rank_row_map, int num_tokens, int num_topk, int num_rows,
+                                float* combined_topk_weights, int64_t* combined_topk_idx) {
+  for (int t = 0; t < num_tokens; ++t)
+    for (int k = 0; k < num_topk; ++k) {
+      size_t i = (size_t)t * num_topk + k;
+      int row = rank_row_map[i];
+      int live = row >= 0 && row < num_rows;
+      if (combined_topk_weights) combined_topk_weights[i] = live ? recv_topk_weights[(size_t)row * num_topk + k] : 0.0f;
+      if (combined_topk_idx) combined_topk_idx[i] = live ? recv_topk_idx[(size_t)row * num_topk + k] : -1;
+    }
+}
+
+/* counts[b, r] = tokens of block b (tile_tokens consecutive tokens) flagged for rank r. */
+int ep_oracle_tile_rank_counts(const uint8_t* is_token_in_rank, int num_tokens, int num_ranks,
+                               int tile_tokens, int* counts) {
+  if (tile_tokens <= 0 || num_ranks <= 0 || num_tokens < 0) return -1;
+  int tiles = (num_tokens + tile_tokens - 1) / tile_tokens;
+  memset(counts, 0, sizeof(int) * (size_t)tiles * num_ranks);
+  for (int t = 0; t < num_tokens; ++t)
+    for (int r = 0; r < num_ranks; ++r)
+      if (is_token_in_rank[(size_t)t * num_ranks + r]) ++counts[(size_t)(t / tile_tokens) * num_ranks + r];
+  return 0;
+}
+
+/* stats[e] += num_tokens_per_expert[e]: the running per-expert totals a caller keeps over launches. */
+void ep_oracle_accumulate_stats(const int* num_tokens_per_expert, int num_experts, int* stats) {
+  for (int e = 0; e < num_experts; ++e) stats[e] += num_tokens_per_expert[e];
 }
 
 /* Per-expert constant scale used by the round-trip workload: rows of expert e are

@@ -251,6 +251,51 @@ def gather_weights(recv_w: np.ndarray, slot_map: np.ndarray) -> np.ndarray:
     return out
 
 
+def gather_idx(recv_idx: np.ndarray, slot_map: np.ndarray) -> np.ndarray:
+    recv_idx = _c(recv_idx, np.int64)
+    slot_map = _c(slot_map, np.int32)
+    T, K = slot_map.shape
+    out = np.empty((T, K), dtype=np.int64)
+    _load().ep_oracle_gather_idx(_p(recv_idx), _p(slot_map), T, K, _p(out))
+    return out
+
+
+def gather_rank_side(recv_w, recv_idx, rank_row_map: np.ndarray):
+    """(combined_topk_weights, combined_topk_idx) of the per-rank format; either input may be None."""
+    rank_row_map = _c(rank_row_map, np.int32)
+    T, K = rank_row_map.shape
+    rows = 0
+    out_w = out_i = None
+    if recv_w is not None:
+        recv_w = _c(recv_w, np.float32)
+        rows = recv_w.shape[0]
+        out_w = np.empty((T, K), dtype=np.float32)
+    if recv_idx is not None:
+        recv_idx = _c(recv_idx, np.int64)
+        rows = recv_idx.shape[0]
+        out_i = np.empty((T, K), dtype=np.int64)
+    _load().ep_oracle_gather_rank_side(_p(recv_w), _p(recv_idx), _p(rank_row_map), T, K, rows, _p(out_w), _p(out_i))
+    return out_w, out_i
+
+
+def tile_rank_counts(flags: np.ndarray, tile_tokens: int = 256) -> np.ndarray:
+    flags = _c(flags, np.uint8)
+    T, R = flags.shape
+    out = np.empty(((T + tile_tokens - 1) // tile_tokens, R), dtype=np.int32)
+    rc = _load().ep_oracle_tile_rank_counts(_p(flags), T, R, tile_tokens, _p(out))
+    if rc != 0:
+        raise ValueError(f"ep_oracle_tile_rank_counts: {rc}")
+    return out
+
+
+def accumulate_stats(per_expert: np.ndarray, stats: np.ndarray) -> np.ndarray:
+    """stats += per_expert, in place; returns stats."""
+    per_expert = _c(per_expert, np.int32)
+    assert stats.dtype == np.int32 and stats.flags.c_contiguous and stats.shape == per_expert.shape
+    _load().ep_oracle_accumulate_stats(_p(per_expert), per_expert.shape[0], _p(stats))
+    return stats
+
+
 def scale_rows_by_expert(rows_bits: np.ndarray, off: np.ndarray, denom: float, num_threads: int = 1):
     rows_bits = _c(rows_bits, np.uint16)
     off = _c(off, np.int32)

@@ -10,6 +10,7 @@
 //
 // Test code: links the CPU checker (oracle/libep_oracle.so) as well as libmi_ep.so.
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 #include <iomanip>
 #include <iostream>
@@ -271,7 +272,20 @@ struct MetricRow {
   double latency_us = 0.0, mtokens_per_s = 0.0;
   int hidden = 0;             // payload rows only
   double data_bytes = 0.0;    // the reference harness's own data-size formula for the row
+  double hbm_bytes = 0.0;     // minimum traffic of the call: every input read once, every output written once
+  bool host_pointers = false; // timed through a host-pointer entry point (transfers and allocation included)
 };
+
+constexpr double kPeakHbmGBps = 8000.0;  // published HBM bandwidth of the part the kernels are written for
+
+// Minimum traffic of the layout calls: the routing table in, flags and counters out
+// (the fused form also writes the offsets, per-route positions and its destination-order table).
+double layout_bytes(const Case& c, bool fused) {
+  const double t = c.tokens, k = c.topk;
+  double b = t * k * 8 + t * c.ranks + (c.ranks + c.experts) * 4.0;
+  if (fused) b += (c.experts + 1) * 4.0 + t * k * 4 + t * k * 16;
+  return b;
+}
 
 template <class Launch>
 MetricRow time_launches(const std::string& surface, const Case& c, Launch launch) {
@@ -302,10 +316,36 @@ void benchmark_case(const Case& c, std::vector<MetricRow>* rows) {
   DeviceArray<bool> d_flags(static_cast<size_t>(c.tokens) * c.ranks);
   d_idx.upload(idx);
   mi_ep::DeepepDispatchLayout layout(c.tokens, c.topk, c.ranks, c.experts);
-  rows->push_back(time_launches("get_dispatch_layout", c, [&] { layout.compute(d_idx.p, d_rank.p, d_expert.p, d_flags.p); }));
+  MetricRow counts = time_launches("get_dispatch_layout", c, [&] { layout.compute(d_idx.p, d_rank.p, d_expert.p, d_flags.p); });
+  counts.hbm_bytes = layout_bytes(c, false);
+  rows->push_back(counts);
   mi_ep::ExpertParallelBuffer buf(c.tokens, c.topk, c.experts, c.ranks);
-  rows->push_back(time_launches("fused_layout", c, [&] { buf.get_dispatch_layout(d_idx.p, c.tokens); }));
+  MetricRow fused = time_launches("fused_layout", c, [&] { buf.get_dispatch_layout(d_idx.p, c.tokens); });
+  fused.hbm_bytes = layout_bytes(c, true);
+  rows->push_back(fused);
   buf.check_status();
+}
+
+// The same layout through the host-pointer twin: what a caller that keeps its data in host vectors
+// pays (allocation, transfers and a synchronisation per call), as the reference's harness does around
+// its kernel (example042 .cu:243-293).
+void benchmark_host_case(const Case& c, std::vector<MetricRow>* rows) {
+  const std::vector<TopkIdx> idx = make_topk(c);
+  std::vector<int> rank(c.ranks), expert(c.experts);
+  std::vector<unsigned char> flags(static_cast<size_t>(c.tokens) * c.ranks);
+  const int iters = 10;
+  const auto t0 = std::chrono::steady_clock::now();
+  for (int i = 0; i < iters; ++i)
+    MI_EP_CHECK(mi_ep_host_get_dispatch_layout(idx.data(), rank.data(), nullptr, expert.data(),
+                                               reinterpret_cast<bool*>(flags.data()), c.tokens, c.topk, c.ranks,
+                                               c.experts));
+  const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count() / iters;
+  MetricRow row{"host_get_dispatch_layout", c};
+  row.latency_us = us;
+  row.mtokens_per_s = us > 0.0 ? c.tokens / us : 0.0;
+  row.hbm_bytes = layout_bytes(c, false);
+  row.host_pointers = true;
+  rows->push_back(row);
 }
 
 // Dispatch (fused layout + permute) and combine at one shape, timed the same way.  data_bytes
@@ -331,10 +371,12 @@ void benchmark_payload_case(const Case& c, int hidden, std::vector<MetricRow>* r
   });
   d.hidden = hidden;
   d.data_bytes = n * 8 + n * 4 + ((c.tokens + 255) / 256) * c.ranks * 4.0;
+  d.hbm_bytes = layout_bytes(c, true) + static_cast<double>(c.tokens) * hidden * 2 + n * hidden * 2 + n * 8 + n * 4 + n * 4;
   rows->push_back(d);
   MetricRow m = time_launches("combine", c, [&] { buf.combine(d_recv.p, buf.capacity_rows(), d_w.p, nullptr, nullptr, hidden, d_out.p); });
   m.hidden = hidden;
   m.data_bytes = n * hidden * 2 + static_cast<double>(c.tokens) * hidden * 2 + n * 4;
+  m.hbm_bytes = n * hidden * 2 + static_cast<double>(c.tokens) * hidden * 2 + n * 4 + n * 4;
   rows->push_back(m);
   buf.check_status();
 }
@@ -350,6 +392,12 @@ void print_json(bool pass, const std::vector<MetricRow>& rows) {
               << ", \"num_ranks\": " << r.c.ranks << ", \"num_experts\": " << r.c.experts << ", \"pattern\": \""
               << pattern_name(r.c.pattern) << "\", \"throughput_avg\": " << r.mtokens_per_s
               << ", \"latency_avg\": " << r.latency_us;
+    {
+      const double gbps = r.latency_us > 0.0 ? r.hbm_bytes / r.latency_us / 1e3 : 0.0;
+      std::cout << ", \"hbm_bytes\": " << r.hbm_bytes << ", \"hbm_gbps\": " << gbps << ", \"roofline_frac\": "
+                << std::setprecision(5) << gbps / kPeakHbmGBps << std::setprecision(3)
+                << ", \"host_pointers\": " << (r.host_pointers ? "true" : "false");
+    }
     if (r.hidden > 0)
       std::cout << ", \"hidden\": " << r.hidden << ", \"data_bytes\": " << r.data_bytes
                 << ", \"gbytes_per_s\": " << (r.latency_us > 0.0 ? r.data_bytes / r.latency_us / 1e3 : 0.0);
@@ -408,6 +456,7 @@ int main(int argc, char** argv) {
     benchmark_case({65536, 4, 8, 32, kRankSweep}, &rows);
     benchmark_case({65536, 8, 8, 32, kSameRank}, &rows);
     benchmark_case({65536, 2, 4, 32, kSpread}, &rows);
+    benchmark_host_case({4096, 2, 8, 32, kSpread}, &rows);
     // The JIT examples' default shape (example080 build_and_run.py:542-548) and the large shape.
     benchmark_payload_case({512, 2, 8, 64, kSpread}, 256, &rows);
     benchmark_payload_case({8192, 8, 8, 256, kSpread}, 7168, &rows);

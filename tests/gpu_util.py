@@ -34,7 +34,8 @@ def garbage_like(t: torch.Tensor) -> torch.Tensor:
 
 
 RANK_SLOT_BASE = 5 * 65536
-SCHEDULE_AUTO, SCHEDULE_BY_TOKEN, SCHEDULE_BY_DESTINATION = 0, 1, 2   # mi_ep_set_dispatch_schedule
+SCHEDULES = ("token", "destination")                                   # both copy kernels (ops.Buffer.dispatch)
+BY_TOKEN, BY_DESTINATION = 2, 4                                        # MI_EP_DISPATCH_BY_* flag bits
 TILE_TOKENS = 256                                                     # tokens per route_order tile
 
 

@@ -32,15 +32,11 @@ def dispatch_and_check(oracle, cfg_or_shape, topk_np, w_np, x_cpu, scales_cpu, a
     ref = oracle.full_path(topk_np, w_np, gu.as_bytes(x_cpu),
                            None if scales_cpu is None else scales_cpu.numpy(), E, R, align)
     rows = int(ref["expert_offsets"][-1])
-    lib = _lib.load()
-    for schedule in (gu.SCHEDULE_BY_TOKEN, gu.SCHEDULE_BY_DESTINATION):
+    for schedule in gu.SCHEDULES:
         print(f"schedule {schedule}", flush=True)
-        assert lib.mi_ep_set_dispatch_schedule(schedule) == 0
-        try:
-            recv_x, recv_scales, recv_src_map, h = buf.dispatch(x, scales, topk, w, expert_alignment=align)
-            torch.cuda.synchronize()
-        finally:
-            assert lib.mi_ep_set_dispatch_schedule(gu.SCHEDULE_AUTO) == 0
+        recv_x, recv_scales, recv_src_map, h = buf.dispatch(x, scales, topk, w, expert_alignment=align,
+                                                            schedule=schedule)
+        torch.cuda.synchronize()
         buf.status()
         assert h.num_recv_rows() == rows
         np.testing.assert_array_equal(h.slot_map.cpu().numpy(), ref["slot_map"])
@@ -121,7 +117,7 @@ def test_alignment_pads_are_zero_rows(oracle, align):
     assert pads.any() and not gu.as_bytes(recv_x)[:off[-1]][pads].any()
 
 
-@pytest.mark.parametrize("schedule", [gu.SCHEDULE_BY_TOKEN, gu.SCHEDULE_BY_DESTINATION])
+@pytest.mark.parametrize("schedule", gu.SCHEDULES)
 def test_scale_factors_through_strides(oracle, schedule):
     """Scale factors in a column-major, padded tensor on the way in and column-major on the way out
     (the reference addresses them through token and hidden strides, example080 .cu:40)."""
@@ -137,14 +133,10 @@ def test_scale_factors_through_strides(oracle, schedule):
     scales_view = padded[:, :T].t()
     assert not scales_view.is_contiguous() and scales_view.stride() == (1, T + 19)
     buf = ops.Buffer(T, K, E, R, device=gu.DEV)
-    lib = _lib.load()
-    assert lib.mi_ep_set_dispatch_schedule(schedule) == 0
-    try:
-        recv_x, recv_scales, _, h = buf.dispatch(xq.to(gu.DEV), scales_view, torch.from_numpy(topk_np).to(gu.DEV),
-                                                 None, expert_alignment=align, column_major_recv_scales=True)
-        torch.cuda.synchronize()
-    finally:
-        assert lib.mi_ep_set_dispatch_schedule(gu.SCHEDULE_AUTO) == 0
+    recv_x, recv_scales, _, h = buf.dispatch(xq.to(gu.DEV), scales_view, torch.from_numpy(topk_np).to(gu.DEV),
+                                             None, expert_alignment=align, column_major_recv_scales=True,
+                                             schedule=schedule)
+    torch.cuda.synchronize()
     ref = oracle.full_path(topk_np, None, gu.as_bytes(xq), scales_cpu.numpy(), E, R, align)
     rows = int(ref["expert_offsets"][-1])
     assert recv_scales.stride()[0] == 1                                    # column-major as asked

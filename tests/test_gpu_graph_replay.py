@@ -13,13 +13,10 @@ from . import gpu_util as gu
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=[gu.SCHEDULE_BY_TOKEN, gu.SCHEDULE_BY_DESTINATION], ids=["by_token", "by_destination"])
+@pytest.fixture(params=[gu.BY_TOKEN, gu.BY_DESTINATION], ids=["by_token", "by_destination"])
 def schedule(request):
-    """Forces one of the two copy kernels for the duration of a test (captured graphs keep it)."""
-    lib = _lib.load()
-    assert lib.mi_ep_set_dispatch_schedule(request.param) == 0
-    yield request.param
-    assert lib.mi_ep_set_dispatch_schedule(gu.SCHEDULE_AUTO) == 0
+    """One of the two copy kernels, as the flag bit mi_ep_dispatch takes."""
+    return request.param
 
 
 def test_graph_replays_match_eager(oracle, schedule):
@@ -51,14 +48,14 @@ def test_graph_replays_match_eager(oracle, schedule):
         _lib.check(lib.mi_ep_dispatch_layout(
             topk.data_ptr(), T, K, R, E, 1, 0, per_rank.data_ptr(), per_expert.data_ptr(),
             in_rank.data_ptr(), off.data_ptr(), psum.data_ptr(), None, slot_rel.data_ptr(), None, 0,
-            route_order.data_ptr(), ws.data_ptr(), ws_bytes, stream), "layout")
+            route_order.data_ptr(), None, None, None, ws.data_ptr(), ws_bytes, stream), "layout")
         _lib.check(lib.mi_ep_dispatch(
             x.data_ptr(), None, topk.data_ptr(), w.data_ptr(), off.data_ptr(), slot_rel.data_ptr(),
             route_order.data_ptr(), per_expert.data_ptr(), T, K, E, 1, H * 2, 0, recv_x.data_ptr(), None, src_map.data_ptr(),
-            recv_idx.data_ptr(), recv_w.data_ptr(), slot_map.data_ptr(), cap, 0, stream), "dispatch")
+            recv_idx.data_ptr(), recv_w.data_ptr(), slot_map.data_ptr(), cap, schedule, stream), "dispatch")
         _lib.check(lib.mi_ep_combine(
-            recv_x.data_ptr(), cap, slot_map.data_ptr(), w.data_ptr(), None, None, None, T, K, H,
-            out.data_ptr(), None, stream), "combine")
+            recv_x.data_ptr(), cap, slot_map.data_ptr(), w.data_ptr(), None, None, None, None, T, K, H,
+            out.data_ptr(), None, None, stream), "combine")
 
     def load_inputs(seed):
         r = np.random.default_rng(seed)
@@ -102,7 +99,8 @@ def test_graph_replays_match_eager(oracle, schedule):
 
 
 def test_two_streams_with_their_own_workspaces(oracle):
-    """Calls are stream-ordered and re-entrant: two buffers on two streams, interleaved launches."""
+    """Calls are stream-ordered and re-entrant: two buffers on two streams, interleaved launches,
+    each stream under its own copy kernel (the choice travels in the call's flags)."""
     E, R, K, H = 64, 8, 8, 512
     rng = np.random.default_rng(77)
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
@@ -119,7 +117,7 @@ def test_two_streams_with_their_own_workspaces(oracle):
     for rep in range(3):
         for i, c in enumerate(cases):
             with torch.cuda.stream(streams[i]):
-                recv_x, _, _, h = c["buf"].dispatch(c["x"], None, c["topk"], c["w"])
+                recv_x, _, _, h = c["buf"].dispatch(c["x"], None, c["topk"], c["w"], schedule=gu.SCHEDULES[i])
                 out = ops.combine(recv_x, h, c["w"])
                 results[i] = (recv_x, h, out)
     torch.cuda.synchronize()

@@ -157,7 +157,7 @@ def test_expired_wait_terminates_and_is_reported(oracle):
     topk = torch.from_numpy(topk_np).to(gu.DEV)
     buf = ops.Buffer(T, K, E, R, device=gu.DEV)
     try:
-        assert lib.mi_ep_set_wait_limit(1) == 0
+        buf.set_wait_limit(1)
         expired = False
         for _ in range(20):                       # every launch terminates; some wait will expire
             buf.dispatch_layout(topk)
@@ -171,7 +171,7 @@ def test_expired_wait_terminates_and_is_reported(oracle):
         with pytest.raises(_lib.MiEpError):
             buf.status()
     finally:
-        assert lib.mi_ep_set_wait_limit(0) == 0
+        buf.set_wait_limit(0)
     _lib.check(lib.mi_ep_workspace_init(buf.workspace.data_ptr(), buf.workspace.numel(),
                                         torch.cuda.current_stream().cuda_stream), "re-init")
     _, h = gu.run_fused_layout(buf, topk_np)

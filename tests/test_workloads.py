@@ -54,3 +54,13 @@ def test_reference_patterns_match_their_formulas():
     assert len(wl.REFERENCE_LAYOUT_CASES) == 13
     f = wl.reference_notify_flags(10, 4, 0)
     assert f.sum() == 20 and f[3, 3] == 1 and f[3, 0] == 1
+
+
+def test_expert_outputs_generated_in_blocks_equal_the_one_shot_generator():
+    """bench.py fills its expert outputs block by block from the same generator stream."""
+    import torch
+    cfg = wl.CONFIGS["c1"]
+    whole = wl.make_expert_outputs(cfg, 300)
+    rng = wl.rng_for(cfg, 2)
+    blocks = torch.cat([wl.bf16_normal(rng, n, cfg.hidden) for n in (128, 128, 44)])
+    assert torch.equal(whole.view(torch.int16), blocks.view(torch.int16))

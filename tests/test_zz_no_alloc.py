@@ -31,10 +31,14 @@ class LayoutOutputs:
         self.rank_slot_idx = torch.full((max(T, 1), K), -3, **i32)
         # entries past the last token are never written: same fill on both sides
         self.route_order = torch.full((max(lib.mi_ep_route_order_bytes(T, K) // 16, 1), 4), -3, **i32)
+        self.tile_rank_counts = torch.full((max((T + 255) // 256, 1), R), -3, **i32)
+        self.copied_topk_idx = torch.full((max(T, 1), K), -3, dtype=torch.int64, device=gu.DEV)
+        self.stats = torch.full((E,), 1000, **i32)          # accumulated into, not overwritten
 
     def tensors(self):
         return [self.per_rank, self.per_expert, self.flags, self.off, self.psum, self.channel_prefix,
-                self.slot_rel, self.rank_slot_idx, self.route_order]
+                self.slot_rel, self.rank_slot_idx, self.route_order, self.tile_rank_counts,
+                self.copied_topk_idx, self.stats]
 
 
 def run_both(lib, topk_np, R, E, align, channels):
@@ -49,12 +53,14 @@ def run_both(lib, topk_np, R, E, align, channels):
         topk.data_ptr(), T, K, R, E, align, channels, want.per_rank.data_ptr(), want.per_expert.data_ptr(),
         want.flags.data_ptr(), want.off.data_ptr(), want.psum.data_ptr(), want.channel_prefix.data_ptr(),
         want.slot_rel.data_ptr(), want.rank_slot_idx.data_ptr(), gu.RANK_SLOT_BASE, want.route_order.data_ptr(),
+        want.tile_rank_counts.data_ptr(), want.copied_topk_idx.data_ptr(), want.stats.data_ptr(),
         ws.data_ptr(), ws_bytes, stream), "mi_ep_dispatch_layout")
     report = torch.zeros(1, dtype=torch.int32, device=gu.DEV)
     _lib.check(lib.mi_ep_dispatch_layout_static(
         topk.data_ptr(), T, K, R, E, align, channels, got.per_rank.data_ptr(), got.per_expert.data_ptr(),
         got.flags.data_ptr(), got.off.data_ptr(), got.psum.data_ptr(), got.channel_prefix.data_ptr(),
         got.slot_rel.data_ptr(), got.rank_slot_idx.data_ptr(), gu.RANK_SLOT_BASE, got.route_order.data_ptr(),
+        got.tile_rank_counts.data_ptr(), got.copied_topk_idx.data_ptr(), got.stats.data_ptr(),
         report.data_ptr(), stream), "mi_ep_dispatch_layout_static")
     torch.cuda.synchronize()
     _lib.check(lib.mi_ep_workspace_status(ws.data_ptr(), stream), "workspace status")
@@ -93,8 +99,8 @@ def test_static_layout_refuses_shapes_beyond_its_scratch():
     # nothing is launched, so no buffer is touched: null outputs are never reached
     one = torch.zeros(8, dtype=torch.int64, device=gu.DEV)
     rc = lib.mi_ep_dispatch_layout_static(one.data_ptr(), T, K, R, E, 1, 0, one.data_ptr(), one.data_ptr(),
-                                          one.data_ptr(), None, None, None, None, None, 0, None, None,
-                                          torch.cuda.current_stream().cuda_stream)
+                                          one.data_ptr(), None, None, None, None, None, 0, None, None, None,
+                                          None, None, torch.cuda.current_stream().cuda_stream)
     assert rc == E2BIG
     assert "static scratch" in _lib.strerror(rc)
     torch.cuda.synchronize()
