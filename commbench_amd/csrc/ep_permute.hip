@@ -39,7 +39,7 @@ constexpr int kDies = 8;
 constexpr int kDieL2BytesMin = 4 * 1024 * 1024;
 constexpr size_t kTileSourceBytesMax = 3840u * 1024u;
 constexpr size_t kRowBytesMin = 4u * 1024u;
-constexpr size_t kFatRowBytesMax = 12u * 1024u;  // below this, 8 KiB instead of 2 KiB per workgroup
+constexpr size_t kRowWideBytesMax = 12u * 1024u;  // up to this, one workgroup per route row instead of 2 KiB parts
 constexpr int kRunRowsMin = 4;
 // The first workgroups of a tile pull its source rows into L2, 8 rows per group of workgroups.
 constexpr int kPrefetchGroups = 32;
@@ -191,8 +191,8 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
 __device__ __forceinline__ void pad_markers_from_prefetch_workgroup(const PermuteArgs& a, const int prefetch_ys,
                                                                     const int rounds) {
   const long long wg = (static_cast<long long>(blockIdx.z) * prefetch_ys + blockIdx.y) * gridDim.x + blockIdx.x;
-  write_pad_markers(a, wg * kPushThreads + static_cast<int>(threadIdx.x),
-                    static_cast<long long>(rounds) * prefetch_ys * gridDim.x * kPushThreads);
+  write_pad_markers(a, wg * blockDim.x + static_cast<int>(threadIdx.x),
+                    static_cast<long long>(rounds) * prefetch_ys * gridDim.x * blockDim.x);
 }
 
 // The same copy in destination order.  A tile is the layout kernel's 256 tokens; its
@@ -208,8 +208,13 @@ __device__ __forceinline__ void pad_markers_from_prefetch_workgroup(const Permut
 // of eight tiles) so that no index needs a division: a wave moves only 1 KiB, which leaves it
 // a budget of about a hundred vector instructions before instruction issue, not HBM, sets the pace.
 // kPads: expert_alignment > 1 (pad markers and pad rounds compiled in); kScales: scale factors travel.
-template <int kVecs, bool kPads, bool kScales>
-__global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const PermuteArgs a, const int num_tiles) {
+// kRowWide: one workgroup of ceil(row / 1 KiB) waves per route instead of two-wave workgroups that
+// each take kVecs KiB-per-wave parts of it: no idle lanes on rows that are not a multiple of the
+// part size (kVecs is 1 then and there is one part).
+template <int kVecs, bool kPads, bool kScales, bool kRowWide>
+__global__ __launch_bounds__(kRowWide ? static_cast<int>(kRowWideBytesMax / sizeof(vec16)) : kPushThreads) void ep_permute_tiles_kernel(const PermuteArgs a,
+                                                                                         const int num_tiles) {
+  static_assert(!kRowWide || kVecs == 1, "a row-wide workgroup moves one vector per lane");
   constexpr int prefetch_ys = kPrefetchGroups;
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
@@ -231,7 +236,8 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
       const vec16 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int u = 0; u < kVecs; ++u) {
-        const int v = (part * kPushWaves + wave) * (kWave * kVecs) + u * kWave + lane;
+        const int v = kRowWide ? static_cast<int>(threadIdx.x)
+                               : (part * kPushWaves + wave) * (kWave * kVecs) + u * kWave + lane;
         if (v < a.row_vecs) __builtin_nontemporal_store(zero, a.recv_x + static_cast<size_t>(row) * a.row_vecs + v);
       }
       return;
@@ -245,7 +251,7 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
     // when the rows come from HBM (not from the memory-side cache) this keeps their reads from
     // being sprinkled over the whole tile, where they would break up the runs of writes
     // (measured at 8192 x 14 KiB rows: 182 us against 208 us; a few us lost when the rows are cached).
-    const int v0 = (part * kPushWaves + wave) * (kWave * kVecs) + lane;
+    const int v0 = kRowWide ? static_cast<int>(threadIdx.x) : (part * kPushWaves + wave) * (kWave * kVecs) + lane;
     constexpr int rows_per_y = kTileTokens / prefetch_ys;
     const int row0 = tile * kTileTokens + static_cast<int>(blockIdx.y) * rows_per_y;
     // Rows past the last token are clamped to it, so that all loads are issued back to back under
@@ -288,7 +294,7 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
   if (flat < first_flat || flat >= first_flat + routes || token < 0 || token >= a.num_tokens) return;
   const bool routed = expert >= 0 && expert < a.num_experts && rel >= 0;
 
-  const int v0 = (part * kPushWaves + wave) * (kWave * kVecs) + lane;
+  const int v0 = kRowWide ? static_cast<int>(threadIdx.x) : (part * kPushWaves + wave) * (kWave * kVecs) + lane;
   vec16 buf[kVecs];
 #pragma unroll
   for (int u = 0; u < kVecs; ++u) {
@@ -328,17 +334,18 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_tiles_kernel(const Pe
   }
 }
 
-template <int kVecs>
-hipError_t launch_permute_tiles(const PermuteArgs& a, const dim3 grid, const int tiles, hipStream_t stream) {
+template <int kVecs, bool kRowWide>
+hipError_t launch_permute_tiles(const PermuteArgs& a, const dim3 grid, const int threads, const int tiles,
+                                hipStream_t stream) {
   const bool pads = a.expert_alignment > 1, scales = a.recv_scales != nullptr;
   if (pads && scales)
-    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, true, true>), grid, dim3(kPushThreads), 0, stream, a, tiles);
+    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, true, true, kRowWide>), grid, dim3(threads), 0, stream, a, tiles);
   else if (pads)
-    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, true, false>), grid, dim3(kPushThreads), 0, stream, a, tiles);
+    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, true, false, kRowWide>), grid, dim3(threads), 0, stream, a, tiles);
   else if (scales)
-    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, false, true>), grid, dim3(kPushThreads), 0, stream, a, tiles);
+    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, false, true, kRowWide>), grid, dim3(threads), 0, stream, a, tiles);
   else
-    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, false, false>), grid, dim3(kPushThreads), 0, stream, a, tiles);
+    hipLaunchKernelGGL((ep_permute_tiles_kernel<kVecs, false, false, kRowWide>), grid, dim3(threads), 0, stream, a, tiles);
   return hipGetLastError();
 }
 
@@ -596,10 +603,6 @@ __global__ __launch_bounds__(256) void ep_write_yardstick_kernel(vec16* __restri
 
 }  // namespace
 
-// Destination order pays when every die has work in (nearly) every round, a tile's rows fit L2,
-// rows are long enough for a workgroup to have something to move and a tile leaves an expert a
-// run of several adjacent rows.  Measured against the token-major kernel, whole copy:
-// 14 KiB rows -13..-16 %, 8 KiB rows -8..-13 %, 4 KiB rows -13 %, 6-7 KiB rows -3..0 %.
 hipError_t device_traits(hipStream_t stream, DeviceTraits* out) {
   // Properties of the hardware, read once per device ordinal and never changed afterwards.
   constexpr int kMaxDevices = 64;
@@ -625,6 +628,11 @@ hipError_t device_traits(hipStream_t stream, DeviceTraits* out) {
   return hipSuccess;
 }
 
+// Destination order pays when every die has work in (nearly) every round, a tile's rows fit L2,
+// rows are long enough for a workgroup to have something to move and a tile leaves an expert a
+// run of several adjacent rows.  Measured against the token-order kernel, whole copy, 8192 tokens,
+// 256 experts, top-8: rows of 4 / 5 / 6 / 7 / 8 / 10 / 12 / 14 KiB: -8 / -9 / -8 / -6 / -13 / -6 / -10 /
+// -11 % (2 KiB rows: +17 %); the same within two points at 4096 and at 16384 tokens.
 bool destination_order_pays(const PermuteArgs& a, const DeviceTraits& dev) {
   // The die mapping and the L2 budget are built into the kernel: any other device takes the token order.
   if (dev.dies != kDies || dev.l2_bytes < kDieL2BytesMin) return false;
@@ -650,10 +658,12 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
   if (by_destination) {
     const int tiles = (a.num_tokens + kTileTokens - 1) / kTileTokens;
     const int rounds = (tiles + kDies - 1) / kDies;
-    // Long rows: 2 KiB per workgroup, seven workgroups on a 14 KiB row.  Short rows do better with
-    // 8 KiB per workgroup (one or two per row): fewer, fatter workgroups for the same bytes.
-    const bool fat = static_cast<size_t>(a.row_vecs) * sizeof(vec16) < kFatRowBytesMax;
-    const int per_workgroup = kPushWaves * kWave * (fat ? 4 : 1);
+    // Long rows: 2 KiB per workgroup, seven workgroups on a 14 KiB row.  Rows up to 12 KiB do better
+    // with one workgroup of ceil(row / 1 KiB) waves each (measured at 8192 tokens, 5 / 6 / 7 / 8 / 10 /
+    // 12 KiB rows: 63 / 75 / 88 / 93 / 122 / 140 us against 66 / 81 / 95 / 96 / 126 / 143 us; 14 KiB
+    // rows: 170 against 166 us).
+    const bool row_wide = static_cast<size_t>(a.row_vecs) * sizeof(vec16) <= kRowWideBytesMax;
+    const int per_workgroup = row_wide ? static_cast<int>(kRowWideBytesMax / sizeof(vec16)) : kPushWaves * kWave;
     const int parts = (a.row_vecs + per_workgroup - 1) / per_workgroup;
     const int prefetch_ys = kPrefetchGroups;
     const int ys = kTileTokens * a.num_topk + prefetch_ys;
@@ -663,7 +673,8 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
     if (rounds + pad_rounds > 65535 || parts * kDies > 65535) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(parts * kDies), static_cast<unsigned>(ys),
                     static_cast<unsigned>(rounds + pad_rounds));
-    return fat ? launch_permute_tiles<4>(a, grid, tiles, stream) : launch_permute_tiles<1>(a, grid, tiles, stream);
+    if (row_wide) return launch_permute_tiles<1, true>(a, grid, (a.row_vecs + kWave - 1) / kWave * kWave, tiles, stream);
+    return launch_permute_tiles<1, false>(a, grid, kPushThreads, tiles, stream);
   }
   const int batches = (a.row_vecs + kWave - 1) / kWave;
   long long units = static_cast<long long>(a.num_tokens) * batches;
