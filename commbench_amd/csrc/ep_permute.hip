@@ -93,8 +93,8 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
   if (token >= a.num_tokens) {
     if (a.expert_alignment <= 1) return;
     // Units past the last token: first the pad rows' side data (one item per lane), then, when the
-    // pads are zeroed, one unit per (pad item, batch) in row order, so that the fill is a linear
-    // stream wherever pad rows are adjacent.
+    // pads are zeroed, one unit per pad item in row order, so that the fill is a linear stream
+    // wherever pad rows are adjacent.
     const long long items = static_cast<long long>(a.num_experts) * (a.expert_alignment - 1);
     const long long marker_units = (items + kWave - 1) / kWave;
     const long long u = unit - static_cast<long long>(a.num_tokens) * batches_per_row;
@@ -103,18 +103,13 @@ __global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteA
       return;
     }
     if (!a.zero_pad_payload) return;
-    const long long z = u - marker_units;
-    const long long item = z / batches_per_row;
+    const long long item = u - marker_units;   // one wave per pad item zeroes the whole row
     if (item >= items) return;
     const int row = pad_row_of_item(a, static_cast<int>(item));
     if (row < 0) return;
-    const int zb = static_cast<int>(z - item * batches_per_row);
     const vec16 zero = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int q = 0; q < kBatchVecs; ++q) {
-      const int v = zb * (kBatchVecs * kWave) + q * kWave + lane;
-      if (v < a.row_vecs) __builtin_nontemporal_store(zero, a.recv_x + static_cast<size_t>(row) * a.row_vecs + v);
-    }
+    vec16* dst = a.recv_x + static_cast<size_t>(row) * a.row_vecs;
+    for (int v = lane; v < a.row_vecs; v += kWave) __builtin_nontemporal_store(zero, dst + v);
     return;
   }
   const int K = a.num_topk;
@@ -227,19 +222,21 @@ __global__ __launch_bounds__(kRowWide ? static_cast<int>(kRowWideBytesMax / size
     if (!kPads) return;
     const int rounds = (num_tiles + kDies - 1) / kDies;  // grid rounds beyond these are pad rounds
     if (static_cast<int>(blockIdx.z) >= rounds) {
-      // Pad rounds (only launched when pad rows are zeroed): workgroup (die, y) of pad round r takes
-      // pad item ((r * gridDim.y + y) * 8 + die), so the dies write adjacent rows side by side.
-      const long long item = (static_cast<long long>(static_cast<int>(blockIdx.z) - rounds) * gridDim.y + blockIdx.y) * kDies + die;
+      // Pad rounds (only launched when pad rows are zeroed): every workgroup takes one pad item and
+      // zeroes that whole row; consecutive workgroups of a die take consecutive rows and the dies'
+      // rows are side by side, so the fill is close to a linear stream wherever pad rows are adjacent.
+      const long long wg = (static_cast<long long>(static_cast<int>(blockIdx.z) - rounds) * gridDim.y + blockIdx.y) * (gridDim.x >> 3) + part;
+      const long long item = wg * kDies + die;
       if (item >= static_cast<long long>(a.num_experts) * (a.expert_alignment - 1)) return;
       const int row = pad_row_of_item(a, static_cast<int>(item));
       if (row < 0) return;
       const vec16 zero = {0u, 0u, 0u, 0u};
-#pragma unroll
-      for (int u = 0; u < kVecs; ++u) {
-        const int v = kRowWide ? static_cast<int>(threadIdx.x)
-                               : (part * kPushWaves + wave) * (kWave * kVecs) + u * kWave + lane;
-        if (v < a.row_vecs) __builtin_nontemporal_store(zero, a.recv_x + static_cast<size_t>(row) * a.row_vecs + v);
-      }
+      vec16* dst = a.recv_x + static_cast<size_t>(row) * a.row_vecs;
+      // Nontemporal stores like the copy's: on its own a fill of these rows is faster with plain
+      // stores (221 MB: 28 us against 43 us), but behind the copy it was not (222 us against 218 us
+      // for the whole kernel), and pad rounds ahead of the copy cost 30 us more than behind it.
+      for (int v = static_cast<int>(threadIdx.x); v < a.row_vecs; v += static_cast<int>(blockDim.x))
+        __builtin_nontemporal_store(zero, dst + v);
       return;
     }
     if (static_cast<int>(blockIdx.y) < prefetch_ys) pad_markers_from_prefetch_workgroup(a, prefetch_ys, rounds);
@@ -667,9 +664,9 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
     const int parts = (a.row_vecs + per_workgroup - 1) / per_workgroup;
     const int prefetch_ys = kPrefetchGroups;
     const int ys = kTileTokens * a.num_topk + prefetch_ys;
-    // Zeroed pads: extra rounds behind the copy, eight pad rows (one per die) per y.
-    const long long pad_rounds =
-        (pad_items > 0 && a.zero_pad_payload) ? (pad_items + static_cast<long long>(ys) * kDies - 1) / (static_cast<long long>(ys) * kDies) : 0;
+    // Zeroed pads: extra rounds behind the copy, one pad row per workgroup.
+    const long long per_pad_round = static_cast<long long>(ys) * kDies * parts;
+    const long long pad_rounds = (pad_items > 0 && a.zero_pad_payload) ? (pad_items + per_pad_round - 1) / per_pad_round : 0;
     if (rounds + pad_rounds > 65535 || parts * kDies > 65535) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(parts * kDies), static_cast<unsigned>(ys),
                     static_cast<unsigned>(rounds + pad_rounds));
@@ -680,7 +677,7 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
   long long units = static_cast<long long>(a.num_tokens) * batches;
   if (pad_items > 0) {
     units += (pad_items + kWave - 1) / kWave;             // side data of the pad rows, one item per lane
-    if (a.zero_pad_payload) units += pad_items * batches;  // their payload, one unit per KiB
+    if (a.zero_pad_payload) units += pad_items;            // their payload, one unit per possible pad row
   }
   const long long blocks = (units + kPushWaves - 1) / kPushWaves;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
