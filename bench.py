@@ -41,6 +41,9 @@ def parse_args():
                     help="skip the PCIe-inclusive pass through the host-pointer entry points")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short runs of the other configurations reported under other_configs")
+    ap.add_argument("--other-configs", default="all",
+                    help="comma-separated names of the other configurations to run (e.g. 'target/ranks,target@128'); "
+                         "default: all of them")
     ap.add_argument("--no-yardsticks", action="store_true",
                     help="skip the linear copy / read / write streams measured beside the roofline")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -537,8 +540,11 @@ def main():
         variants = [("c2", 1, 0), ("c3", 1, 0), ("c4", 1, 0), ("c5", 1, 0), ("target", 1, 0),
                     (cfg.name + "@128", 128, 0), (cfg.name + "@128/keep", 128, KEEP_PAD_PAYLOAD),
                     (cfg.name + "/ranks", 1, 0)]
+        wanted = None if args.other_configs == "all" else set(args.other_configs.split(","))
+        if wanted is not None and not wanted <= {v[0] for v in variants}:
+            sys.exit(f"--other-configs: unknown name(s) {sorted(wanted - {v[0] for v in variants})}")
         for name, align, flags in variants:
-            if name == cfg.name:
+            if name == cfg.name or (wanted is not None and name not in wanted):
                 continue
             ocfg = wl.CONFIGS[name.split("@")[0].split("/")[0]]
             ranks_format = name.endswith("/ranks")

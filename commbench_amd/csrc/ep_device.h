@@ -58,6 +58,7 @@ struct LayoutArgs {
   int expert_alignment;
   int num_channels;
   int num_tiles;
+  int static_tiles;  // 1: workgroup b takes tile b (every workgroup is resident at once); 0: tiles by ticket
   int rank_slot_base;
   int expert_bits;  // ceil(log2(num_experts)), at least 1
   uint32_t inv_topk;              // ceil(2^19 / num_topk): n / num_topk == (n * inv) >> 19 for n < 2048

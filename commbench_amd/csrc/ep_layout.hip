@@ -83,8 +83,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   const int cols = E + R;
   int* col_total = smem;                    // [cols] this tile's total per column
   int* col_excl = col_total + cols;         // [cols] sum over earlier tiles
-  int* rank_cnt = col_excl + cols;          // [kMaxRanks]
-  int* wave_sums = rank_cnt + kMaxRanks;    // [kLayoutWaves]
+  int* wave_sums = col_excl + cols;         // [kLayoutWaves]
   int* misc = wave_sums + kLayoutWaves;     // [4] tile, generation, wait limit
   int* rank_wave = misc + 4;                // [kTileTokens / kWave][kMaxRanks] flagged tokens per wave
   int* order_sums = rank_wave + (kTileTokens / kWave) * kMaxRanks;  // [kLayoutWaves] scan of the tile's counts
@@ -98,6 +97,31 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   const int wave = tid >> 6;
   uint64_t* status = reinterpret_cast<uint64_t*>(a.ws + 1);
 
+  // ---- routes: the tile's 256*K routes are 4*K chunks of 64 in (token, slot)
+  // order; wave w owns chunks [w * per_wave, (w + 1) * per_wave).
+  const int flat_end = T * K;
+  const int num_chunks = (kTileTokens / kWave) * K;
+  const int per_wave = (num_chunks + kLayoutWaves - 1) / kLayoutWaves;  // <= kChunksPerWave
+  int64_t raw[kChunksPerWave];
+  auto load_routes = [&](const int of_tile) {
+#pragma unroll
+    for (int c = 0; c < kChunksPerWave; ++c) {
+      raw[c] = -1;
+      const int chunk = wave * per_wave + c;
+      if (c < per_wave && chunk < num_chunks) {
+        const int g = of_tile * (kTileTokens * K) + chunk * kWave + lane;
+        if (g < flat_end) {
+          raw[c] = a.topk_idx[g];
+          if (a.copied_topk_idx != nullptr) a.copied_topk_idx[g] = raw[c];
+        }
+      }
+    }
+  };
+
+  // One fetch-add per tile on the workspace's turn word: its high half is the launch's generation,
+  // its low half counts arrivals; the last arrival hands the workspace to the next launch.  The
+  // arrival number is also the tile unless tiles are static, in which case the routes are fetched
+  // while the fetch-add is still on its way.
   if (tid == 0) {
     const uint64_t turn =
         __hip_atomic_fetch_add(&a.ws->turn, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -107,45 +131,27 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     misc[1] = static_cast<int>(generation);
     const uint32_t limit = a.ws->wait_limit;
     misc[2] = static_cast<int>(limit != 0 ? limit : kDefaultWaitLimit);
-    // Last ticket of the launch: hand the workspace to the next launch.
     if (ticket == static_cast<uint32_t>(a.num_tiles) - 1u)
       __hip_atomic_store(&a.ws->turn, static_cast<uint64_t>((generation + 1u) & kGenMask) << 32,
                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  if (a.static_tiles) load_routes(static_cast<int>(blockIdx.x));
   {
     uint32_t* hist_words = reinterpret_cast<uint32_t*>(hist);
     for (int i = tid; i < (kLayoutWaves * E + 1) / 2; i += kLayoutThreads) hist_words[i] = 0;
   }
-  if (tid < kMaxRanks) rank_cnt[tid] = 0;
   if (tid < kTileTokens) tok_flags[tid] = 0;
   __syncthreads();
 
-  const int tile = misc[0];
+  const int tile = a.static_tiles ? static_cast<int>(blockIdx.x) : misc[0];
   const uint32_t gen = static_cast<uint32_t>(misc[1]);
   const uint32_t wait_limit = static_cast<uint32_t>(misc[2]);
   if (tile >= a.num_tiles) return;  // stale ticket: never with an initialised workspace
   const int t0 = tile * kTileTokens;
   const int flat0 = t0 * K;
-  const int flat_end = T * K;
   uint16_t* my_hist = hist + wave * E;
+  if (!a.static_tiles) load_routes(tile);
 
-  // ---- routes: the tile's 256*K routes are 4*K chunks of 64 in (token, slot)
-  // order; wave w owns chunks [w * per_wave, (w + 1) * per_wave).
-  const int num_chunks = (kTileTokens / kWave) * K;
-  const int per_wave = (num_chunks + kLayoutWaves - 1) / kLayoutWaves;  // <= kChunksPerWave
-  int64_t raw[kChunksPerWave];
-#pragma unroll
-  for (int c = 0; c < kChunksPerWave; ++c) {
-    raw[c] = -1;
-    const int chunk = wave * per_wave + c;
-    if (c < per_wave && chunk < num_chunks) {
-      const int g = flat0 + chunk * kWave + lane;
-      if (g < flat_end) {
-        raw[c] = a.topk_idx[g];
-        if (a.copied_topk_idx != nullptr) a.copied_topk_idx[g] = raw[c];
-      }
-    }
-  }
   int my_e[kChunksPerWave];
   int my_pos[kChunksPerWave];  // rank among the wave's earlier routes to the same expert (among its non-routes if masked)
   int masked_seen = 0;
@@ -183,17 +189,23 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   if (lane == 0) masked_wave[wave] = masked_seen;
   __syncthreads();
 
-  // ---- expert columns: wave bases, tile total, aggregate published at once ------
-  // (the status words need a few microseconds to reach the other tiles; the flag
-  // pass and the scan for the tile's route order run in that shadow)
+  // ---- every column's aggregate is published as early as possible: the status words need a
+  // microsecond or two to become visible to the other tiles, and a look-back that polls before
+  // its predecessors' words have landed pays a whole extra round trip.  Everything that does not
+  // need the look-back's result runs between the publication and the first poll.
+  // Expert columns (thread e < E): wave bases, tile total, aggregate out.
   int my_col_total = 0;  // thread e < E: this tile's routes to expert e
   for (int col = tid; col < E; col += kLayoutThreads) {
+    // All reads before the first write: as one read-modify-write chain the sixteen LDS round trips
+    // would run one after the other.
+    int v[kLayoutWaves];
+#pragma unroll
+    for (int w = 0; w < kLayoutWaves; ++w) v[w] = hist[w * E + col];
     int total = 0;
 #pragma unroll
     for (int w = 0; w < kLayoutWaves; ++w) {
-      const int v = hist[w * E + col];
       hist[w * E + col] = static_cast<uint16_t>(total);  // becomes the wave's base inside the tile
-      total += v;
+      total += v[w];
     }
     col_total[col] = total;
     my_col_total = total;
@@ -211,43 +223,97 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     }
     if (lane == kWave - 1) order_sums[wave] = order_incl;
   }
-
-  // ---- flags out, de-duplicated rank hits (one token per thread) ---------------
-  if (tid < kTileTokens) {
-    const int t = t0 + tid;
-    const uint64_t f = tok_flags[tid];
-    if (t < T) store_token_flags(a.is_token_in_rank, t, R, f);
-    for (int r = 0; r < R; ++r) {
-      const uint64_t hit = __ballot(((f >> (8 * r)) & 1u) != 0);
-      if (lane == 0 && hit != 0) atomicAdd(&rank_cnt[r], __popcll(hit));
+  // Rank hits, de-duplicated per token: one token per thread of waves 4..7 (the waves next to the
+  // ones that hold the expert columns of up to 256 experts).  below_packed, byte r: flagged tokens
+  // of rank r in this wave before this token, kept for the slot table after the look-back.  The
+  // token's ids for that table are fetched here and folded into four bits per slot further down,
+  // so that little state stays in registers across the look-back.
+  const int ftid = tid - kTileTokens;           // token of the tile, on the flag threads
+  const bool flag_thread = ftid >= 0 && ftid < kTileTokens;
+  const int fwave = ftid >> 6;                  // 0..3 on the flag threads
+  uint64_t my_flags = 0, below_packed = 0;
+  int64_t my_ids[kMaxTopk];
+#pragma unroll
+  for (int k = 0; k < kMaxTopk; ++k) my_ids[k] = -1;
+  if (flag_thread) {  // whole waves
+    if (a.rank_slot_idx != nullptr && t0 + ftid < T) {
+#pragma unroll
+      for (int k = 0; k < kMaxTopk; ++k)
+        if (k < K) my_ids[k] = a.topk_idx[static_cast<size_t>(t0 + ftid) * K + k];
+    }
+    my_flags = tok_flags[ftid];
+#pragma unroll
+    for (int r = 0; r < kMaxRanks; ++r) {
+      const uint64_t hit = __ballot(r < R && ((my_flags >> (8 * r)) & 1u) != 0);
+      below_packed |= static_cast<uint64_t>(__popcll(hit & lanes_below(lane))) << (8 * r);
+      if (lane == 0) rank_wave[fwave * kMaxRanks + r] = __popcll(hit);
     }
   }
   __syncthreads();
 
+  // Rank columns (thread r < R): the tile's total out.
+  if (tid < R) {
+    int total = 0;
+#pragma unroll
+    for (int w = 0; w < kTileTokens / kWave; ++w) total += rank_wave[w * kMaxRanks + tid];
+    col_total[E + tid] = total;
+    publish(status + static_cast<size_t>(tile) * cols + E + tid,
+            pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
+    if (a.tile_rank_counts != nullptr) a.tile_rank_counts[static_cast<size_t>(tile) * R + tid] = total;
+  }
+  // In the shadow of the publication: the flags go out and the cross-wave half of the route-order
+  // scan is folded in.
+  if (flag_thread && t0 + ftid < T) store_token_flags(a.is_token_in_rank, t0 + ftid, R, my_flags);
   int masked_base = 0;  // where this wave's non-routes start in the tile's route order
   if (a.route_order != nullptr) {
+    // Unconditional reads, selected afterwards, so that they are issued together.
+    int sums[kLayoutWaves], masked[kLayoutWaves];
+#pragma unroll
+    for (int w = 0; w < kLayoutWaves; ++w) {
+      sums[w] = order_sums[w];
+      masked[w] = masked_wave[w];
+    }
     int base = order_incl - my_col_total;
 #pragma unroll
     for (int w = 0; w < kLayoutWaves; ++w) {
-      if (w < wave) base += order_sums[w];
-      masked_base += order_sums[w];  // every route of the tile comes first
-      if (w < wave) masked_base += masked_wave[w];
+      base += (w < wave) ? sums[w] : 0;
+      masked_base += sums[w] + ((w < wave) ? masked[w] : 0);  // every route of the tile comes first
     }
-    if (tid < E) offs[tid] = base;  // read after the barrier that ends the look-back
+    if (tid < E) offs[tid] = base;
+  }
+  __syncthreads();
+
+  // Each route's place inside the tile (needs the wave bases and the scan, not the look-back).
+  int in_tile[kChunksPerWave], order_pos[kChunksPerWave];
+#pragma unroll
+  for (int c = 0; c < kChunksPerWave; ++c) {
+    const int e = my_e[c];
+    in_tile[c] = (e >= 0) ? my_hist[e] + my_pos[c] : 0;
+    order_pos[c] = (a.route_order == nullptr) ? 0 : (e >= 0) ? offs[e] + in_tile[c] : masked_base + my_pos[c];
   }
 
-  // ---- rank columns published, then the decoupled look-back of every column ------
-  for (int col = tid; col < cols; col += kLayoutThreads) {
-    int total;
-    uint64_t* mine = status + static_cast<size_t>(tile) * cols + col;
-    if (col < E) {
-      total = col_total[col];
-    } else {
-      total = rank_cnt[col - E];
-      col_total[col] = total;
-      if (a.tile_rank_counts != nullptr) a.tile_rank_counts[static_cast<size_t>(tile) * R + (col - E)] = total;
-      publish(mine, pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
+  // Slot k of the token opens a row of rank r when it is the first slot that reaches r: nibble k
+  // of first_ranks holds 8 | r then, 0 otherwise.
+  uint32_t first_ranks = 0;
+  if (flag_thread && a.rank_slot_idx != nullptr) {
+    uint32_t seen = 0;
+#pragma unroll
+    for (int k = 0; k < kMaxTopk; ++k) {
+      const int64_t e64 = my_ids[k];
+      if (k < K && e64 >= 0 && e64 < static_cast<int64_t>(E)) {
+        const uint32_t rank = (static_cast<uint32_t>(e64) * a.inv_experts_per_rank) >> 22;
+        if (((seen >> rank) & 1u) == 0) {
+          seen |= 1u << rank;
+          first_ranks |= (8u | rank) << (4 * k);
+        }
+      }
     }
+  }
+
+  // ---- the decoupled look-back of every column ----------------------------------
+  for (int col = tid; col < cols; col += kLayoutThreads) {
+    const int total = col_total[col];
+    uint64_t* mine = status + static_cast<size_t>(tile) * cols + col;
     int excl = 0;
     if (tile != 0) {
       // Fold predecessors in, nearest first, a window of independent loads at a
@@ -257,6 +323,8 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
       uint32_t spins = 0;
       bool found_prefix = false;
       while (!found_prefix) {
+        // Only rows that exist are fetched: every row costs about 0.1 us (33 uncached 64-byte
+        // sectors per row and tile), far more than the branch around its load.
         uint64_t s[kLookbackWindow];
 #pragma unroll
         for (int i = 0; i < kLookbackWindow; ++i) {
@@ -308,13 +376,11 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
         const int g = flat0 + local;
         if (g < flat_end) {
           const int e = my_e[c];
-          const int in_tile = (e >= 0) ? my_hist[e] + my_pos[c] : 0;
-          const int rel = (e >= 0) ? col_excl[e] + in_tile : -1;
+          const int rel = (e >= 0) ? col_excl[e] + in_tile[c] : -1;
           if (a.slot_rel != nullptr) a.slot_rel[g] = rel;
           if (a.route_order != nullptr) {
             const int token = t0 + static_cast<int>((static_cast<uint32_t>(local) * a.inv_topk) >> 19);
-            const int pos = (e >= 0) ? offs[e] + in_tile : masked_base + my_pos[c];
-            order[pos] = make_int4(g, e, rel, token);
+            order[order_pos[c]] = make_int4(g, e, rel, token);
           }
         }
       }
@@ -323,43 +389,26 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
 
   // ---- the deterministic prologue's table: per destination rank, tokens take slots in
   // token order; the first slot of a token that reaches the rank carries the slot number
-  if (a.rank_slot_idx != nullptr) {
-    int below[kMaxRanks];
-    uint64_t f = 0;
-    if (tid < kTileTokens) {
-      f = tok_flags[tid];
+  if (a.rank_slot_idx != nullptr && flag_thread && t0 + ftid < T) {
+    int position[kMaxRanks];
 #pragma unroll
-      for (int r = 0; r < kMaxRanks; ++r) {
-        const uint64_t hit = __ballot(r < R && ((f >> (8 * r)) & 1u) != 0);
-        below[r] = __popcll(hit & lanes_below(lane));
-        if (lane == 0) rank_wave[wave * kMaxRanks + r] = __popcll(hit);
+    for (int r = 0; r < kMaxRanks; ++r) {
+      int base = col_excl[E + (r < R ? r : 0)];
+#pragma unroll
+      for (int w = 0; w < kTileTokens / kWave - 1; ++w) {
+        const int before = rank_wave[w * kMaxRanks + r];  // read by every wave, counted by the later ones
+        base += (w < fwave) ? before : 0;
       }
+      position[r] = a.rank_slot_base + base + static_cast<int>((below_packed >> (8 * r)) & 0xffu);
     }
-    __syncthreads();
-    const int t = t0 + tid;
-    if (tid < kTileTokens && t < T) {
-      int position[kMaxRanks];
 #pragma unroll
-      for (int r = 0; r < kMaxRanks; ++r) {
-        int base = r < R ? col_excl[E + r] : 0;
-        for (int w = 0; w < wave; ++w) base += rank_wave[w * kMaxRanks + r];
-        position[r] = a.rank_slot_base + base + below[r];
-      }
-      uint32_t seen = 0;
-      for (int k = 0; k < K; ++k) {
-        const int64_t e64 = a.topk_idx[static_cast<size_t>(t) * K + k];
+    for (int k = 0; k < kMaxTopk; ++k) {
+      if (k < K) {
+        const uint32_t nibble = (first_ranks >> (4 * k)) & 0xfu;
         int out = -1;
-        if (e64 >= 0 && e64 < static_cast<int64_t>(E)) {
-          const int rank = static_cast<int>((static_cast<uint32_t>(e64) * a.inv_experts_per_rank) >> 22);
-          if (((seen >> rank) & 1u) == 0) {
-            seen |= 1u << rank;
-            int slot = 0;
 #pragma unroll
-            for (int r = 0; r < kMaxRanks; ++r) slot = (r == rank) ? position[r] : slot;
-            out = slot;
-          }
-        }
-        a.rank_slot_idx[static_cast<size_t>(t) * K + k] = out;
+        for (int r = 0; r < kMaxRanks; ++r) out = (nibble == (8u | r)) ? position[r] : out;
+        a.rank_slot_idx[static_cast<size_t>(t0 + ftid) * K + k] = out;
       }
     }
   }
@@ -414,8 +463,9 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
       int grand = 0;
 #pragma unroll
       for (int w = 0; w < kLayoutWaves; ++w) {
-        if (w < wave) base += wave_sums[w];
-        grand += wave_sums[w];
+        const int sum = wave_sums[w];
+        base += (w < wave) ? sum : 0;
+        grand += sum;
       }
       if (tid < E) {
         offs[tid] = base;
@@ -525,7 +575,7 @@ hipError_t launch_layout_fused(const LayoutArgs& a, hipStream_t stream) {
   static_assert(kMaxExperts <= kLayoutThreads, "the offset scan takes one expert per thread");
   const int E = a.num_experts;
   const int cols = E + a.num_ranks;
-  const size_t lds = sizeof(int) * (2 * static_cast<size_t>(cols) + kMaxRanks + kLayoutWaves + 4 +
+  const size_t lds = sizeof(int) * (2 * static_cast<size_t>(cols) + kLayoutWaves + 4 +
                                     (kTileTokens / kWave) * kMaxRanks + 2 * kLayoutWaves + E + 2 + (E & 1)) +
                      sizeof(uint64_t) * kTileTokens + sizeof(uint16_t) * (static_cast<size_t>(kLayoutWaves) * E + 2);
   hipLaunchKernelGGL(ep_layout_fused_kernel, dim3(a.num_tiles), dim3(kLayoutThreads), lds, stream, a);
