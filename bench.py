@@ -47,6 +47,9 @@ def parse_args():
     ap.add_argument("--no-yardsticks", action="store_true",
                     help="skip the linear copy / read / write streams measured beside the roofline")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--schedule-sweep", action="store_true",
+                    help="instead of the benchmark: time the dispatch copy under both schedules over a grid of row "
+                         "sizes and token counts (the table the automatic choice is derived from) and print it as JSON")
     return ap.parse_args()
 
 
@@ -349,8 +352,49 @@ def kernel_medians(torch, wk, reps):
     return marks
 
 
+def schedule_sweep():
+    """Median duration of the dispatch copy inside the running step (layout, dispatch, combine back to
+    back), forced to the token order and to the destination order, for rows of 2-16 KiB."""
+    import torch
+    from commbench_amd import ops, workloads as wl
+    torch.cuda.set_device(0)
+
+    def measure(cfg, flag):
+        wk = Workload(cfg, "cuda:0", dispatch_flags=flag)
+        for _ in range(60):
+            wk.step()
+        torch.cuda.synchronize()
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(40)]
+        for a, b in ev:
+            wk.layout()
+            a.record()
+            wk.dispatch()
+            b.record()
+            wk.combine()
+        torch.cuda.synchronize()
+        t = sorted(a.elapsed_time(b) * 1e3 for a, b in ev)
+        return t[len(t) // 2]
+
+    rows = []
+    for T, E in ((8192, 256), (4096, 256), (16384, 128)):
+        for row_bytes in (2048, 4096, 5120, 6144, 7168, 8192, 10240, 12288, 14336, 16384):
+            cfg = wl.Config(f"sweep{T}_{row_bytes}", 40, T, row_bytes // 2, E, 8, 8)
+            _EXPERT_OUTPUTS.clear()
+            by_token = measure(cfg, ops.BY_TOKEN)
+            by_destination = measure(cfg, ops.BY_DESTINATION)
+            rows.append({"num_tokens": T, "num_experts": E, "row_bytes": row_bytes,
+                         "by_token_us": round(by_token, 1), "by_destination_us": round(by_destination, 1),
+                         "change_pct": round((by_destination / by_token - 1) * 100, 1),
+                         "automatic": ops.dispatch_schedule_for(T, 8, E, row_bytes)})
+            print(json.dumps(rows[-1]), file=sys.stderr, flush=True)
+    print(json.dumps({"schedule_sweep": rows, "device_traits": ops.device_traits()}))
+
+
 def main():
     args = parse_args()
+    if args.schedule_sweep:
+        schedule_sweep()
+        return
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported "
               "(this path has no multi-GPU leg; partitions of one GPU's HBM stand for ranks)",
@@ -404,7 +448,7 @@ def main():
                 wk.stream = torch.cuda.current_stream().cuda_stream
                 wk.step()
         wk.stream = torch.cuda.current_stream().cuda_stream
-        for _ in range(3):
+        for _ in range(30):      # the capture left the device idle: back to sustained clocks first
             graph.replay()
         torch.cuda.synchronize()
         t0 = time.perf_counter()

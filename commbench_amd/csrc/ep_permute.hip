@@ -628,8 +628,9 @@ hipError_t device_traits(hipStream_t stream, DeviceTraits* out) {
 // Destination order pays when every die has work in (nearly) every round, a tile's rows fit L2,
 // rows are long enough for a workgroup to have something to move and a tile leaves an expert a
 // run of several adjacent rows.  Measured against the token-order kernel, whole copy, 8192 tokens,
-// 256 experts, top-8: rows of 4 / 5 / 6 / 7 / 8 / 10 / 12 / 14 KiB: -8 / -9 / -8 / -6 / -13 / -6 / -10 /
-// -11 % (2 KiB rows: +17 %); the same within two points at 4096 and at 16384 tokens.
+// 256 experts, top-8: rows of 4 / 5 / 6 / 7 / 8 / 10 / 12 / 14 KiB: -9 / -8 / -10 / -10 / -13 / -6 / -9 /
+// -11 % (2 KiB rows: +11 %; 16 KiB rows, whose tile no longer fits: -4 %); within five points of that
+// at 4096 tokens and at 16384 tokens with 128 experts, where 16 KiB rows gain nothing.
 bool destination_order_pays(const PermuteArgs& a, const DeviceTraits& dev) {
   // The die mapping and the L2 budget are built into the kernel: any other device takes the token order.
   if (dev.dies != kDies || dev.l2_bytes < kDieL2BytesMin) return false;

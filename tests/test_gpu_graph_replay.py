@@ -100,7 +100,7 @@ def test_graph_replays_match_eager(oracle, schedule):
 
 def test_two_streams_with_their_own_workspaces(oracle):
     """Calls are stream-ordered and re-entrant: two buffers on two streams, interleaved launches,
-    each stream under its own copy kernel (the choice travels in the call's flags)."""
+    each stream under its own copy kernel (the choice travels in the call's flags) and wait limit."""
     E, R, K, H = 64, 8, 8, 512
     rng = np.random.default_rng(77)
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
@@ -112,6 +112,7 @@ def test_two_streams_with_their_own_workspaces(oracle):
         cases.append(dict(T=T, topk_np=topk_np, w_np=w_np, x_cpu=x_cpu, buf=ops.Buffer(T, K, E, R, device=gu.DEV),
                           topk=torch.from_numpy(topk_np).to(gu.DEV), w=torch.from_numpy(w_np).to(gu.DEV),
                           x=x_cpu.to(gu.DEV)))
+    cases[1]["buf"].set_wait_limit(1 << 20)   # a limit of its own, too: it lives in the buffer's workspace
     torch.cuda.synchronize()
     results = [None, None]
     for rep in range(3):
