@@ -205,6 +205,23 @@ def test_permute_random_shapes(oracle, seed):
     dispatch_and_check(oracle, (E, R), topk_np, w_np, x_cpu, scales_cpu, align=align)
 
 
+@pytest.mark.parametrize("shape", [
+    # T, K, E, R, row_bytes, num_scales, alignment: rows on both sides of every workgroup shape of the
+    # destination-order kernel (one workgroup of up to twelve waves per row; 2 KiB parts above 12 KiB)
+    (700, 8, 32, 8, 5136, 3, 1), (700, 8, 32, 8, 12288, 0, 16), (520, 8, 32, 8, 12304, 5, 1),
+    (520, 4, 16, 4, 14352, 0, 128), (300, 8, 16, 8, 20000, 2, 3), (900, 8, 64, 8, 4096, 32, 128)],
+    ids=lambda s: "x".join(map(str, s)))
+def test_permute_row_sizes_around_the_workgroup_shapes(oracle, shape):
+    T, K, E, R, row_bytes, S, align = shape
+    print(f"shape {shape}", flush=True)
+    rng = np.random.default_rng(sum(shape))
+    topk_np = rng.integers(-1, E, size=(T, K)).astype(np.int64)
+    w_np = rng.standard_normal((T, K)).astype(np.float32)
+    x_cpu = torch.from_numpy(rng.integers(0, 256, size=(T, row_bytes), dtype=np.uint8))
+    scales_cpu = torch.from_numpy(rng.standard_normal((T, S)).astype(np.float32)) if S else None
+    dispatch_and_check(oracle, (E, R), topk_np, w_np, x_cpu, scales_cpu, align=align)
+
+
 def test_capacity_limits_writes(oracle):
     """Rows at or beyond capacity_rows are dropped: never written, slot_map = -1."""
     rng = np.random.default_rng(3)
