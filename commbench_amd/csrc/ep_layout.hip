@@ -120,22 +120,31 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
 
   // One fetch-add per tile on the workspace's turn word: its high half is the launch's generation,
   // its low half counts arrivals; the last arrival hands the workspace to the next launch.  The
-  // arrival number is also the tile unless tiles are static, in which case the routes are fetched
-  // while the fetch-add is still on its way.
+  // arrival number is also the tile unless tiles are static; then nothing needs the fetch-add's
+  // answer before the aggregates are published, so it travels while the routes are fetched and
+  // ranked, and thread 0 hands the generation out just before the barrier that ends the ranking.
+  uint64_t turn = 0;
+  uint32_t limit = 0;
   if (tid == 0) {
-    const uint64_t turn =
-        __hip_atomic_fetch_add(&a.ws->turn, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const uint32_t ticket = static_cast<uint32_t>(turn);
-    const uint32_t generation = static_cast<uint32_t>(turn >> 32) & kGenMask;
-    misc[0] = static_cast<int>(ticket);
-    misc[1] = static_cast<int>(generation);
-    const uint32_t limit = a.ws->wait_limit;
-    misc[2] = static_cast<int>(limit != 0 ? limit : kDefaultWaitLimit);
-    if (ticket == static_cast<uint32_t>(a.num_tiles) - 1u)
-      __hip_atomic_store(&a.ws->turn, static_cast<uint64_t>((generation + 1u) & kGenMask) << 32,
-                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    turn = __hip_atomic_fetch_add(&a.ws->turn, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    limit = a.ws->wait_limit;
   }
-  if (a.static_tiles) load_routes(static_cast<int>(blockIdx.x));
+  auto hand_out = [&]() {
+    if (tid == 0) {
+      const uint32_t ticket = static_cast<uint32_t>(turn);
+      const uint32_t generation = static_cast<uint32_t>(turn >> 32) & kGenMask;
+      misc[0] = static_cast<int>(ticket);
+      misc[1] = static_cast<int>(generation);
+      misc[2] = static_cast<int>(limit != 0 ? limit : kDefaultWaitLimit);
+      if (ticket == static_cast<uint32_t>(a.num_tiles) - 1u)
+        __hip_atomic_store(&a.ws->turn, static_cast<uint64_t>((generation + 1u) & kGenMask) << 32,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+  if (a.static_tiles)
+    load_routes(static_cast<int>(blockIdx.x));
+  else
+    hand_out();
   {
     uint32_t* hist_words = reinterpret_cast<uint32_t*>(hist);
     for (int i = tid; i < (kLayoutWaves * E + 1) / 2; i += kLayoutThreads) hist_words[i] = 0;
@@ -144,8 +153,6 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   __syncthreads();
 
   const int tile = a.static_tiles ? static_cast<int>(blockIdx.x) : misc[0];
-  const uint32_t gen = static_cast<uint32_t>(misc[1]);
-  const uint32_t wait_limit = static_cast<uint32_t>(misc[2]);
   if (tile >= a.num_tiles) return;  // stale ticket: never with an initialised workspace
   const int t0 = tile * kTileTokens;
   const int flat0 = t0 * K;
@@ -187,7 +194,10 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     }
   }
   if (lane == 0) masked_wave[wave] = masked_seen;
+  if (a.static_tiles) hand_out();
   __syncthreads();
+  const uint32_t gen = static_cast<uint32_t>(misc[1]);
+  const uint32_t wait_limit = static_cast<uint32_t>(misc[2]);
 
   // ---- every column's aggregate is published as early as possible: the status words need a
   // microsecond or two to become visible to the other tiles, and a look-back that polls before
