@@ -192,6 +192,20 @@ __device__ __forceinline__ int lane_id() { return static_cast<int>(threadIdx.x) 
 
 __device__ __forceinline__ uint64_t lanes_below(int lane) { return (1ull << lane) - 1ull; }
 
+// Inclusive prefix sum over the 64 lanes of a wave with data-parallel-primitive moves (no LDS
+// round trips as a shuffle would take): shifts by 1, 2, 4, 8 inside each row of 16 lanes (lanes
+// without a source add the 0 given as the old value), then the last lane of row 0 / 2 into rows 1 / 3
+// and lane 31 into rows 2 and 3.
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // Value of `v` in lane `src` (wave-uniform src), as a scalar.
 __device__ __forceinline__ int wave_read(int v, int src) {
   return __builtin_amdgcn_readlane(v, src);

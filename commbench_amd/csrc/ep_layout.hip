@@ -226,11 +226,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   // routes start in the tile's route order.  The cross-wave half follows the next barrier.
   int order_incl = my_col_total;
   if (a.route_order != nullptr) {
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const int up = __shfl_up(order_incl, d, kWave);
-      if (lane >= d) order_incl += up;
-    }
+    order_incl = wave_inclusive_scan(my_col_total);
     if (lane == kWave - 1) order_sums[wave] = order_incl;
   }
   // Rank hits, de-duplicated per token: one token per thread of waves 4..7 (the waves next to the
@@ -461,12 +457,7 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
         const int cnt = col_excl[tid] + col_total[tid];
         local = (cnt + align - 1) / align * align;
       }
-      int incl = local;
-#pragma unroll
-      for (int d = 1; d < kWave; d <<= 1) {
-        const int up = __shfl_up(incl, d, kWave);
-        if (lane >= d) incl += up;
-      }
+      const int incl = wave_inclusive_scan(local);
       if (lane == kWave - 1) wave_sums[wave] = incl;
       __syncthreads();
       int base = incl - local;
