@@ -469,16 +469,13 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
         grand += sum;
       }
       if (tid < E) {
-        offs[tid] = base;
         a.expert_offsets[tid] = base;
+        // The thread of a rank's last expert holds the rank's inclusive row count.
+        const int rank_end = static_cast<int>((static_cast<uint32_t>(tid + 1) * a.inv_experts_per_rank) >> 22);
+        if (a.psum_rank_rows != nullptr && rank_end * a.experts_per_rank == tid + 1)
+          a.psum_rank_rows[rank_end - 1] = base + local;
       }
-      if (tid == 0) {
-        offs[E] = grand;
-        a.expert_offsets[E] = grand;
-      }
-      __syncthreads();
-      if (a.psum_rank_rows != nullptr && tid < R)
-        a.psum_rank_rows[tid] = offs[(tid + 1) * a.experts_per_rank];
+      if (tid == 0) a.expert_offsets[E] = grand;
     }
   }
 }
