@@ -147,11 +147,15 @@ int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, in
   a.expert_alignment = expert_alignment;
   a.num_channels = num_channels;
   a.num_tiles = num_tiles_for(num_tokens);
-  // With at most one workgroup per compute unit every tile is resident at once, so the look-back can
-  // never wait on a tile that has not started and the tiles need no tickets (one memory round trip
-  // less before the first load).  Larger grids take tickets, which orders the tiles by arrival.
+  // Small grids take static tiles (workgroup b = tile b: one memory round trip less before the first
+  // load).  A look-back then may wait on a tile whose workgroup has not started, which is harmless as
+  // long as that workgroup finds a slot: with at most one tile per eight compute units a launch takes
+  // 1/16 of the slots its workgroups could occupy (two fit a compute unit), so that sixteen such
+  // launches would have to execute at once, each partly resident, before one could keep another's
+  // tiles out -- more than a process has hardware queues.  Larger grids take tickets, which order the
+  // tiles by arrival and need no such argument.  The wait is bounded either way.
   DeviceTraits dev{};
-  a.static_tiles = (device_traits(s, &dev) == hipSuccess && a.num_tiles <= dev.compute_units) ? 1 : 0;
+  a.static_tiles = (device_traits(s, &dev) == hipSuccess && a.num_tiles * 8 <= dev.compute_units) ? 1 : 0;
   a.expert_bits = 1;
   while ((1 << a.expert_bits) < num_experts) ++a.expert_bits;
   a.inv_topk = ((1u << 19) + num_topk - 1) / num_topk;
