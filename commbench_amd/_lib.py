@@ -49,6 +49,9 @@ SIGNATURES = {
                                           _vp, _vp, _int, _vp, _vp, _vp, _vp]),
     "mi_ep_host_dispatch": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _int,
                                    _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int]),
+    "mi_ep_host_dispatch_ranks": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _int, _int,
+                                         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int]),
+    "mi_ep_host_dispatch_cached": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp, _vp]),
     "mi_ep_host_combine": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
     "mi_ep_copy_yardstick": (_int, [_vp, _vp, _size, _vp]),
     "mi_ep_read_yardstick": (_int, [_vp, _size, _vp, _vp]),

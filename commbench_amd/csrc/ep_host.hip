@@ -226,6 +226,102 @@ int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* top
   return s.status(MI_EP_OK);
 }
 
+int mi_ep_host_dispatch_ranks(const void* x, const float* x_scales, const int64_t* topk_idx,
+                              const float* topk_weights, int num_tokens, int num_topk, int num_ranks,
+                              int num_experts, int row_bytes, int num_scales, int source_token_base,
+                              int local_expert_ids, int* num_tokens_per_rank, void* recv_x,
+                              float* recv_scales, int64_t* recv_topk_idx, float* recv_topk_weights,
+                              int* recv_src_metadata, int* rank_row_map, int* combine_map,
+                              int* psum_rank_tokens, int capacity_rows) {
+  if (num_tokens < 0 || num_topk <= 0 || num_ranks <= 0 || num_experts <= 0) return MI_EP_EINVAL;
+  if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
+  if (psum_rank_tokens == nullptr) return MI_EP_EINVAL;
+  if (num_tokens > 0 && (x == nullptr || topk_idx == nullptr || rank_row_map == nullptr)) return MI_EP_EINVAL;
+  if (capacity_rows > 0 && recv_x == nullptr) return MI_EP_EINVAL;
+  if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
+  if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
+  const size_t workspace_bytes = mi_ep_workspace_bytes(num_tokens > 0 ? num_tokens : 1, num_topk, num_experts, num_ranks);
+  if (workspace_bytes == 0) return MI_EP_EINVAL;
+
+  Staging s;
+  const size_t tk = static_cast<size_t>(num_tokens) * num_topk;
+  const size_t tr = static_cast<size_t>(num_tokens) * num_ranks;
+  const size_t cap = static_cast<size_t>(capacity_rows);
+  const size_t meta = static_cast<size_t>(2 + num_topk);
+  const unsigned char* d_x = s.upload(static_cast<const unsigned char*>(x), static_cast<size_t>(num_tokens) * row_bytes);
+  const float* d_scales = num_scales > 0 ? s.upload(x_scales, static_cast<size_t>(num_tokens) * num_scales) : nullptr;
+  const int64_t* d_topk = s.upload(topk_idx, tk);
+  const float* d_w = s.upload(topk_weights, tk);
+  int* d_rank = s.alloc<int>(num_ranks);
+  int* d_expert = s.alloc<int>(num_experts);
+  bool* d_flags = s.alloc<bool>(tr);
+  int* d_rank_slots = s.alloc<int>(tk);
+  unsigned char* d_ws = s.alloc<unsigned char>(workspace_bytes);
+  unsigned char* d_recv_x = s.alloc<unsigned char>(cap * row_bytes);
+  float* d_recv_scales = num_scales > 0 ? s.alloc<float>(cap * num_scales) : nullptr;
+  int64_t* d_recv_idx = recv_topk_idx != nullptr ? s.alloc<int64_t>(cap * num_topk) : nullptr;
+  float* d_recv_w = recv_topk_weights != nullptr ? s.alloc<float>(cap * num_topk) : nullptr;
+  int* d_meta = recv_src_metadata != nullptr ? s.alloc<int>(cap * meta) : nullptr;
+  int* d_row_map = s.alloc<int>(tk);
+  int* d_combine_map = combine_map != nullptr ? s.alloc<int>(tk) : nullptr;
+  int* d_psum = s.alloc<int>(num_ranks);
+  if (!s.ok()) return s.status(MI_EP_OK);
+
+  int code = mi_ep_workspace_init(d_ws, workspace_bytes, nullptr);
+  if (code == MI_EP_OK)
+    code = mi_ep_dispatch_layout(d_topk, num_tokens, num_topk, num_ranks, num_experts, 1, 0, d_rank, d_expert,
+                                 d_flags, nullptr, nullptr, nullptr, nullptr, d_rank_slots, 0, nullptr, nullptr,
+                                 nullptr, nullptr, d_ws, workspace_bytes, nullptr);
+  if (code == MI_EP_OK)
+    code = mi_ep_dispatch_ranks(d_x, d_scales, d_topk, d_w, d_rank_slots, 0, d_rank, nullptr, num_tokens,
+                                num_topk, num_ranks, num_experts, row_bytes, num_scales, source_token_base,
+                                local_expert_ids, d_recv_x, d_recv_scales, d_recv_idx, d_recv_w, d_meta,
+                                d_row_map, d_combine_map, d_psum, capacity_rows, nullptr);
+  if (code == MI_EP_OK) code = mi_ep_workspace_status(d_ws, nullptr);  // synchronises
+  if (code != MI_EP_OK) return code;
+
+  int total = 0;
+  s.download(&total, d_psum + (num_ranks - 1), 1);
+  if (!s.ok()) return s.status(MI_EP_OK);
+  const size_t rows = static_cast<size_t>(total) < cap ? static_cast<size_t>(total) : cap;
+  s.download(num_tokens_per_rank, d_rank, num_ranks);
+  s.download(static_cast<unsigned char*>(recv_x), d_recv_x, rows * row_bytes);
+  if (num_scales > 0) s.download(recv_scales, d_recv_scales, rows * num_scales);
+  s.download(recv_topk_idx, d_recv_idx, rows * num_topk);
+  s.download(recv_topk_weights, d_recv_w, rows * num_topk);
+  s.download(recv_src_metadata, d_meta, rows * meta);
+  s.download(rank_row_map, d_row_map, tk);
+  s.download(combine_map, d_combine_map, tk);
+  s.download(psum_rank_tokens, d_psum, num_ranks);
+  return s.status(MI_EP_OK);
+}
+
+int mi_ep_host_dispatch_cached(const void* x, const float* x_scales, const int* recv_src_map, int num_rows,
+                               int num_tokens, int row_bytes, int num_scales, void* recv_x,
+                               float* recv_scales) {
+  if (num_rows < 0 || num_tokens < 0 || row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0)
+    return MI_EP_EINVAL;
+  if (num_rows > 0 && (recv_src_map == nullptr || recv_x == nullptr)) return MI_EP_EINVAL;
+  if (num_rows > 0 && num_tokens > 0 && x == nullptr) return MI_EP_EINVAL;
+  if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
+  if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
+  Staging s;
+  const size_t rows = static_cast<size_t>(num_rows);
+  const unsigned char* d_x = s.upload(static_cast<const unsigned char*>(x), static_cast<size_t>(num_tokens) * row_bytes);
+  const float* d_scales = num_scales > 0 ? s.upload(x_scales, static_cast<size_t>(num_tokens) * num_scales) : nullptr;
+  const int* d_map = s.upload(recv_src_map, rows);
+  unsigned char* d_recv_x = s.alloc<unsigned char>(rows * row_bytes);
+  float* d_recv_scales = num_scales > 0 ? s.alloc<float>(rows * num_scales) : nullptr;
+  if (!s.ok()) return s.status(MI_EP_OK);
+  int code = mi_ep_dispatch_cached(d_x, d_scales, d_map, num_rows, num_tokens, row_bytes, num_scales, d_recv_x,
+                                   d_recv_scales, nullptr, 0, nullptr);
+  code = sync_status(code);
+  if (code != MI_EP_OK) return code;
+  s.download(static_cast<unsigned char*>(recv_x), d_recv_x, rows * row_bytes);
+  if (num_scales > 0) s.download(recv_scales, d_recv_scales, rows * num_scales);
+  return s.status(MI_EP_OK);
+}
+
 int mi_ep_host_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
                        const void* bias_0, const void* bias_1, int num_tokens, int num_topk, int hidden,
                        void* combined_x) {

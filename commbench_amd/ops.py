@@ -14,7 +14,8 @@ split into `num_ranks` partitions:
         -> (recv_x, recv_topk_idx, recv_topk_weights, handle)            format: one row per token
     combine_ranks(y, handle, recv_topk_weights) -> combined_x[, weights]  and destination rank
     dispatch_cached / pull_indices                                        pull form from a source map
-    host_get_dispatch_layout / host_dispatch_layout / host_dispatch / host_combine    numpy in, numpy out
+    host_get_dispatch_layout / host_dispatch_layout / host_dispatch / host_dispatch_ranks /
+    host_dispatch_cached / host_combine                                   numpy in, numpy out
 
 torch is used for device memory and streams only; all arithmetic runs in the HIP kernels of
 libmi_ep.so.  Nothing here falls back to torch ops or to the CPU.
@@ -599,6 +600,62 @@ def host_dispatch(x, scales, topk_idx, topk_weights, num_experts: int, num_ranks
         if out[key] is not None:
             out[key] = out[key][:rows]
     return out
+
+
+def host_dispatch_ranks(x, scales, topk_idx, topk_weights, num_experts: int, num_ranks: int,
+                        source_token_base: int = 0, local_expert_ids: bool = False):
+    """Layout + dispatch in the reference's per-rank receive format on host arrays: a dict with
+    num_tokens_per_rank, psum_rank_tokens, rank_row_map, combine_map and the recv_* arrays trimmed to
+    psum_rank_tokens[-1] rows."""
+    import numpy as np
+    topk_idx = _np(topk_idx, np.int64)
+    T, K = topk_idx.shape
+    x = np.ascontiguousarray(x)
+    _require(x.ndim == 2 and x.shape[0] == T, "x must be [num_tokens, row]")
+    row_bytes = x.shape[1] * x.itemsize
+    scales = _np(scales, np.float32)
+    topk_weights = _np(topk_weights, np.float32)
+    S = 0 if scales is None else scales.shape[1]
+    cap = T * min(K, num_ranks)
+    out = dict(
+        num_tokens_per_rank=np.empty(num_ranks, dtype=np.int32),
+        recv_x=np.empty((cap, x.shape[1]), dtype=x.dtype),
+        recv_scales=None if scales is None else np.empty((cap, S), dtype=np.float32),
+        recv_topk_idx=np.empty((cap, K), dtype=np.int64),
+        recv_topk_weights=np.empty((cap, K), dtype=np.float32),
+        recv_src_metadata=np.empty((cap, 2 + K), dtype=np.int32),
+        rank_row_map=np.empty((T, K), dtype=np.int32),
+        combine_map=np.empty((T, K), dtype=np.int32),
+        psum_rank_tokens=np.empty(num_ranks, dtype=np.int32))
+    _lib.check(_lib.load().mi_ep_host_dispatch_ranks(
+        _np_ptr(x), _np_ptr(scales), _np_ptr(topk_idx), _np_ptr(topk_weights), T, K, num_ranks, num_experts,
+        row_bytes, S, source_token_base, 1 if local_expert_ids else 0, _np_ptr(out["num_tokens_per_rank"]),
+        _np_ptr(out["recv_x"]), _np_ptr(out["recv_scales"]), _np_ptr(out["recv_topk_idx"]),
+        _np_ptr(out["recv_topk_weights"]), _np_ptr(out["recv_src_metadata"]), _np_ptr(out["rank_row_map"]),
+        _np_ptr(out["combine_map"]), _np_ptr(out["psum_rank_tokens"]), cap), "mi_ep_host_dispatch_ranks")
+    rows = int(out["psum_rank_tokens"][-1])
+    for key in ("recv_x", "recv_scales", "recv_topk_idx", "recv_topk_weights", "recv_src_metadata"):
+        if out[key] is not None:
+            out[key] = out[key][:rows]
+    return out
+
+
+def host_dispatch_cached(x, scales, recv_src_map):
+    """Pull-form dispatch on host arrays: row i of the result is x[recv_src_map[i]] (zeros where the
+    map holds -1), scales likewise."""
+    import numpy as np
+    recv_src_map = _np(recv_src_map, np.int32)
+    x = np.ascontiguousarray(x)
+    _require(x.ndim == 2 and recv_src_map.ndim == 1, "x must be [num_tokens, row], recv_src_map [num_rows]")
+    T, rows = x.shape[0], recv_src_map.shape[0]
+    scales = _np(scales, np.float32)
+    S = 0 if scales is None else scales.shape[1]
+    recv_x = np.empty((rows, x.shape[1]), dtype=x.dtype)
+    recv_scales = None if scales is None else np.empty((rows, S), dtype=np.float32)
+    _lib.check(_lib.load().mi_ep_host_dispatch_cached(
+        _np_ptr(x), _np_ptr(scales), _np_ptr(recv_src_map), rows, T, x.shape[1] * x.itemsize, S,
+        _np_ptr(recv_x), _np_ptr(recv_scales)), "mi_ep_host_dispatch_cached")
+    return recv_x, recv_scales
 
 
 def host_combine(y_bits, slot_map, topk_weights=None, bias_0=None, bias_1=None):

@@ -364,6 +364,13 @@ int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float*
  *                                   may be NULL) and expert_offsets come back with the permuted
  *                                   rows; only the first min(expert_offsets[E], capacity_rows)
  *                                   rows of the recv_* arrays are written
+ *   mi_ep_host_dispatch_ranks       layout + mi_ep_dispatch_ranks in one call (the reference's own
+ *                                   receive format, example081 .cu:22-60): num_tokens_per_rank (may
+ *                                   be NULL), the per-row arrays (recv_topk_idx, recv_topk_weights,
+ *                                   recv_src_metadata: any may be NULL), rank_row_map, combine_map
+ *                                   (may be NULL) and psum_rank_tokens come back; only the first
+ *                                   min(psum_rank_tokens[R-1], capacity_rows) rows are written
+ *   mi_ep_host_dispatch_cached      twin of mi_ep_dispatch_cached (without arrival counters)
  *   mi_ep_host_combine              twin of mi_ep_combine (without the travelled weights)
  */
 int mi_ep_host_get_dispatch_layout(const int64_t* topk_idx, int* num_tokens_per_rank,
@@ -383,6 +390,16 @@ int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* top
                         int* expert_offsets, void* recv_x, float* recv_scales, int* recv_src_map,
                         int64_t* recv_topk_idx, float* recv_topk_weights, int* slot_map,
                         int capacity_rows);
+int mi_ep_host_dispatch_ranks(const void* x, const float* x_scales, const int64_t* topk_idx,
+                              const float* topk_weights, int num_tokens, int num_topk, int num_ranks,
+                              int num_experts, int row_bytes, int num_scales, int source_token_base,
+                              int local_expert_ids, int* num_tokens_per_rank, void* recv_x,
+                              float* recv_scales, int64_t* recv_topk_idx, float* recv_topk_weights,
+                              int* recv_src_metadata, int* rank_row_map, int* combine_map,
+                              int* psum_rank_tokens, int capacity_rows);
+int mi_ep_host_dispatch_cached(const void* x, const float* x_scales, const int* recv_src_map, int num_rows,
+                               int num_tokens, int row_bytes, int num_scales, void* recv_x,
+                               float* recv_scales);
 int mi_ep_host_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
                        const void* bias_0, const void* bias_1, int num_tokens, int num_topk, int hidden,
                        void* combined_x);

@@ -106,6 +106,9 @@ def test_host_only_entry_points():
     assert lib.mi_ep_host_dispatch(None, None, None, None, 4, 2, 2, 8, 1, 24, 0, None, None, None, None,
                                    None, None, None, None, None, None, 0) == -22
     assert lib.mi_ep_host_combine(None, 0, None, None, None, None, 4, 2, 12, None) == -22
+    assert lib.mi_ep_host_dispatch_ranks(None, None, None, None, 4, 2, 2, 8, 24, 0, 0, 0, None, None, None,
+                                         None, None, None, None, None, None, 0) == -22       # 24 % 16, no psum
+    assert lib.mi_ep_host_dispatch_cached(None, None, None, 4, 4, 24, 0, None, None) == -22
     assert lib.mi_ep_workspace_bytes(8192, 8, 256, 9) == 0       # more than 8 ranks
     assert lib.mi_ep_workspace_bytes(8192, 9, 256, 8) == 0       # more than 8 slots
     assert lib.mi_ep_workspace_bytes(8192, 8, 250, 8) == 0       # experts not divisible by ranks

@@ -58,3 +58,42 @@ def test_host_dispatch_fp8_rows_with_scales(oracle):
     np.testing.assert_array_equal(got["recv_x"], ref["recv_x"])
     np.testing.assert_array_equal(got["recv_scales"].view(np.uint32), ref["recv_scales"].view(np.uint32))
     np.testing.assert_array_equal(got["slot_map"], ref["slot_map"])
+
+
+@pytest.mark.parametrize("local_ids", [False, True])
+def test_host_dispatch_ranks_then_the_plain_sum(oracle, local_ids):
+    """The per-rank receive format through host arrays: every output against the checker, then the
+    reference's combine of that format (ordered sum over combine_map) on the rows it produced."""
+    rng = np.random.default_rng(31)
+    T, K, E, R, H = 700, 8, 32, 8, 256
+    topk = rng.integers(-1, E, size=(T, K)).astype(np.int64)     # masks and duplicates included
+    w = wl.softmax_gates(rng, T, K)
+    x_bits = gu.bf16_bits(wl.bf16_normal(rng, T, H))
+    scales = rng.standard_normal((T, 3)).astype(np.float32)
+    got = ops.host_dispatch_ranks(x_bits, scales, topk, w, E, R, source_token_base=5 * T, local_expert_ids=local_ids)
+    ref = oracle.permute_ranks(x_bits.view(np.uint8), scales, topk, w, R, E, 5 * T, local_ids, None)
+    np.testing.assert_array_equal(got["psum_rank_tokens"], ref["psum_rank_tokens"])
+    np.testing.assert_array_equal(got["num_tokens_per_rank"], oracle.layout(topk, R, E)[0])
+    np.testing.assert_array_equal(got["rank_row_map"], ref["rank_row_map"])
+    first = oracle.rank_slots(topk, R, E, 0) >= 0
+    np.testing.assert_array_equal(got["combine_map"], np.where(first, ref["rank_row_map"], -1))
+    np.testing.assert_array_equal(got["recv_x"].view(np.uint8), ref["recv_x"])
+    np.testing.assert_array_equal(got["recv_scales"].view(np.uint32), ref["recv_scales"].view(np.uint32))
+    np.testing.assert_array_equal(got["recv_topk_idx"], ref["recv_topk_idx"])
+    np.testing.assert_array_equal(got["recv_topk_weights"].view(np.uint32), ref["recv_topk_weights"].view(np.uint32))
+    np.testing.assert_array_equal(got["recv_src_metadata"], ref["recv_src_metadata"])
+    out = ops.host_combine(got["recv_x"], got["combine_map"], None)
+    want = oracle.combine(got["recv_x"], got["combine_map"], None)
+    assert gu.bf16_ulp_distance(out, want).max() <= 2
+
+
+def test_host_dispatch_cached_pulls_rows_by_the_source_map(oracle):
+    rng = np.random.default_rng(32)
+    T, H, rows = 333, 264, 900
+    x_bits = gu.bf16_bits(wl.bf16_normal(rng, T, H))
+    scales = rng.standard_normal((T, 2)).astype(np.float32)
+    src_map = rng.integers(-1, T, size=rows).astype(np.int32)
+    recv_x, recv_scales = ops.host_dispatch_cached(x_bits, scales, src_map)
+    want_x, want_scales = oracle.gather_rows(x_bits.view(np.uint8), scales, src_map)
+    np.testing.assert_array_equal(recv_x.view(np.uint8), want_x)
+    np.testing.assert_array_equal(recv_scales.view(np.uint32), want_scales.view(np.uint32))
