@@ -21,7 +21,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBPS = 8000.0      # MI355X published HBM3E bandwidth
-KEEP_PAD_PAYLOAD = 1        # MI_EP_DISPATCH_KEEP_PAD_PAYLOAD
+ZERO_PAD_PAYLOAD = 1        # MI_EP_DISPATCH_ZERO_PAD_PAYLOAD
 
 
 def parse_args():
@@ -127,7 +127,7 @@ class Workload:
         # the algorithmic count.
         counts = wl.np.bincount(topk_np[topk_np >= 0].ravel(), minlength=E)
         pad_rows = int(((counts + expert_alignment - 1) // expert_alignment * expert_alignment - counts).sum())
-        zeroed = expert_alignment > 1 and not (dispatch_flags & KEEP_PAD_PAYLOAD)
+        zeroed = expert_alignment > 1 and bool(dispatch_flags & ZERO_PAD_PAYLOAD)
         self.pad_rows = pad_rows
         self.padded_bytes = pad_rows * (cfg.row_bytes + cfg.num_scales * 4) if zeroed else 0
 
@@ -577,12 +577,13 @@ def main():
         torch.cuda.empty_cache()
         others = {}
         # "<name>@128": the same shape with expert segments padded to 128 rows, as the reference's
-        # harness asks of dispatch (example080 build_and_run.py:718).  With zero-filled pads the fill
-        # is extra traffic (padded_bytes) on top of the algorithmic count; "@128/keep" leaves the pad
-        # payload alone, which is what the reference's receive buffer does.
+        # harness asks of dispatch (example080 build_and_run.py:718); the pad rows' map entries are
+        # written, their payload is left alone, as in the reference's receive buffer.
+        # "<name>@128/zero": the pad payload zero-filled as well; the fill is extra traffic
+        # (padded_bytes) on top of the algorithmic count.
         # "<name>/ranks": the reference's per-rank receive format.
         variants = [("c2", 1, 0), ("c3", 1, 0), ("c4", 1, 0), ("c5", 1, 0), ("target", 1, 0),
-                    (cfg.name + "@128", 128, 0), (cfg.name + "@128/keep", 128, KEEP_PAD_PAYLOAD),
+                    (cfg.name + "@128", 128, 0), (cfg.name + "@128/zero", 128, ZERO_PAD_PAYLOAD),
                     (cfg.name + "/ranks", 1, 0)]
         wanted = None if args.other_configs == "all" else set(args.other_configs.split(","))
         if wanted is not None and not wanted <= {v[0] for v in variants}:

@@ -310,7 +310,7 @@ int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long lon
   if ((num_scales > 0) != (recv_scales != nullptr)) return MI_EP_EINVAL;
   if (num_scales > 0 && num_tokens > 0 && x_scales == nullptr) return MI_EP_EINVAL;
   if (expert_alignment > 1 && num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
-  if ((flags & ~(MI_EP_DISPATCH_KEEP_PAD_PAYLOAD | kScheduleFlags)) != 0) return MI_EP_EINVAL;
+  if ((flags & ~(MI_EP_DISPATCH_ZERO_PAD_PAYLOAD | kScheduleFlags)) != 0) return MI_EP_EINVAL;
   if ((flags & kScheduleFlags) == kScheduleFlags) return MI_EP_EINVAL;  // one copy kernel at most
   if ((flags & MI_EP_DISPATCH_BY_DESTINATION) != 0 && route_order == nullptr && num_tokens > 0)
     return MI_EP_EINVAL;
@@ -346,7 +346,7 @@ int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long lon
   a.rs_token_stride = recv_scales_token_stride;
   a.rs_hidden_stride = recv_scales_hidden_stride;
   a.expert_alignment = expert_alignment;
-  a.zero_pad_payload = (flags & MI_EP_DISPATCH_KEEP_PAD_PAYLOAD) == 0 ? 1 : 0;
+  a.zero_pad_payload = (flags & MI_EP_DISPATCH_ZERO_PAD_PAYLOAD) != 0 ? 1 : 0;
   const int schedule = (flags & MI_EP_DISPATCH_BY_TOKEN) != 0         ? kPermuteByToken
                        : (flags & MI_EP_DISPATCH_BY_DESTINATION) != 0 ? kPermuteByDestination
                                                                       : kPermuteAuto;

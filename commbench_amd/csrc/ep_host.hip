@@ -205,7 +205,8 @@ int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* top
   if (code == MI_EP_OK)
     code = mi_ep_dispatch(d_x, d_scales, d_topk, d_w, d_off, d_slot_rel, d_order, d_expert, num_tokens,
                           num_topk, num_experts, expert_alignment, row_bytes, num_scales, d_recv_x,
-                          d_recv_scales, d_src_map, d_recv_idx, d_recv_w, d_slot_map, capacity_rows, 0, nullptr);
+                          d_recv_scales, d_src_map, d_recv_idx, d_recv_w, d_slot_map, capacity_rows,
+                          MI_EP_DISPATCH_ZERO_PAD_PAYLOAD, nullptr);  // pad rows come back as zeros
   if (code == MI_EP_OK) code = mi_ep_workspace_status(d_ws, nullptr);  // synchronises
   if (code != MI_EP_OK) return code;
 

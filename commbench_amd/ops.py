@@ -30,7 +30,7 @@ from . import _lib
 MAX_RANKS = 8
 MAX_TOPK = 8
 MAX_EXPERTS = 1024
-KEEP_PAD_PAYLOAD = 1   # MI_EP_DISPATCH_KEEP_PAD_PAYLOAD
+ZERO_PAD_PAYLOAD = 1   # MI_EP_DISPATCH_ZERO_PAD_PAYLOAD
 BY_TOKEN = 2           # MI_EP_DISPATCH_BY_TOKEN
 BY_DESTINATION = 4     # MI_EP_DISPATCH_BY_DESTINATION
 _SCHEDULE_FLAGS = {"auto": 0, "token": BY_TOKEN, "destination": BY_DESTINATION}
@@ -201,13 +201,14 @@ class Buffer:
                  topk_weights: Optional[torch.Tensor], expert_alignment: int = 1,
                  num_channels: int = 0, handle: Optional[DispatchHandle] = None,
                  capacity_rows: Optional[int] = None, rank_slot_base: Optional[int] = None,
-                 zero_pads: bool = True, column_major_recv_scales: bool = False, schedule: str = "auto"):
+                 zero_pads: bool = False, column_major_recv_scales: bool = False, schedule: str = "auto"):
         """Layout (unless `handle` is given) + permute into the expert-contiguous buffer.
 
         Returns (recv_x, recv_scales, recv_src_map, handle).  Buffers hold `capacity_rows` rows
         (default: the worst case T*K + E*(alignment-1), so no host sync is needed); rows at and
-        beyond handle.num_recv_rows() are unspecified.  With expert_alignment > 1 the pad rows are
-        zero rows unless `zero_pads` is False (then only their map entries are written).
+        beyond handle.num_recv_rows() are unspecified.  With expert_alignment > 1 the pad rows'
+        map entries are written (source -1); their payload is left alone, as in the reference's
+        receive buffer, unless `zero_pads` asks for zero rows.
         `scales` may be any 2-D float32 view (row- or column-major, padded); with
         `column_major_recv_scales` the returned recv_scales is a [capacity, S] view of a [S, capacity]
         allocation, the layout the reference's TMA-aligned scale tensors have.
@@ -253,7 +254,7 @@ class Buffer:
             _ptr(handle.num_tokens_per_expert), T, K, E, handle.expert_alignment, row_bytes, num_scales,
             _ptr(recv_x), _ptr(recv_scales), rs_strides[0], rs_strides[1], _ptr(handle.recv_src_map),
             _ptr(handle.recv_topk_idx), _ptr(handle.recv_topk_weights), _ptr(handle.slot_map), capacity_rows,
-            (0 if zero_pads else KEEP_PAD_PAYLOAD) | _SCHEDULE_FLAGS[schedule], _stream()),
+            (ZERO_PAD_PAYLOAD if zero_pads else 0) | _SCHEDULE_FLAGS[schedule], _stream()),
             "mi_ep_dispatch_strided_scales")
         return recv_x, recv_scales, handle.recv_src_map, handle
 

@@ -186,15 +186,16 @@ size_t mi_ep_route_order_bytes(int num_tokens, int num_topk);
  *   recv_topk_idx     int64[capacity_rows] or NULL: expert owning the row; -1 pad
  *   recv_topk_weights float[capacity_rows] or NULL: gate weight of the row's route; 0 pad
  *   slot_map     int32[num_tokens, num_topk]: absolute row of each route, -1 non-routes
- * Rows >= capacity_rows are never written.  With expert_alignment > 1 pad rows are
- * zero-filled by further workgroups of the same launch; num_tokens_per_expert (from the layout
- * call) locates them and may be NULL when expert_alignment == 1.
+ * Rows >= capacity_rows are never written.  With expert_alignment > 1 the pad rows' map entries
+ * are written (source -1, expert -1, weight 0) by further workgroups of the same launch; their
+ * payload and scales are left untouched, as the reference's receive buffer is (its harness pads to
+ * 128 rows and only reads the received ones, example080 build_and_run.py:718,728-748).
+ * num_tokens_per_expert (from the layout call) locates the pad rows and may be NULL when
+ * expert_alignment == 1.
  *   flags        0, or an OR of
- *                MI_EP_DISPATCH_KEEP_PAD_PAYLOAD  leave the payload and scales of pad rows untouched,
- *                  as the reference's receive buffer is (its harness pads to 128 rows and only reads
- *                  the received ones, example080 build_and_run.py:718,728-748); their map entries are
- *                  still written (source -1, expert -1, weight 0).  At alignment 128 the zero fill is
- *                  a fifth of the copy's bytes.
+ *                MI_EP_DISPATCH_ZERO_PAD_PAYLOAD  also zero-fill the payload and scales of pad rows,
+ *                  for consumers that read whole aligned segments.  At alignment 128 the fill is a
+ *                  fifth of the copy's bytes.
  *                MI_EP_DISPATCH_BY_TOKEN / MI_EP_DISPATCH_BY_DESTINATION  (at most one) the copy
  *                  kernel to use instead of the one chosen by shape and device; by destination needs
  *                  route_order.  Results are identical.
@@ -204,7 +205,7 @@ size_t mi_ep_route_order_bytes(int num_tokens, int num_topk);
  *                die that owns the tile), which the HBM write path takes ~14 % faster than
  *                rows scattered token by token.
  */
-#define MI_EP_DISPATCH_KEEP_PAD_PAYLOAD 1
+#define MI_EP_DISPATCH_ZERO_PAD_PAYLOAD 1
 #define MI_EP_DISPATCH_BY_TOKEN 2
 #define MI_EP_DISPATCH_BY_DESTINATION 4
 int mi_ep_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,

@@ -184,7 +184,7 @@ class ExpertParallelBuffer {
   }
 
   // Layout + permute.  recv_x / recv_scales hold capacity_rows() rows; scales may be null.
-  // flags: MI_EP_DISPATCH_* (pad payload kept, copy kernel forced).
+  // flags: MI_EP_DISPATCH_* (pad payload zeroed, copy kernel forced).
   const DispatchHandle& dispatch(const void* d_x, const float* d_scales, const TopkIdx* d_topk_idx,
                                  const float* d_topk_weights, int num_tokens, int row_bytes, int num_scales,
                                  void* d_recv_x, float* d_recv_scales, hipStream_t stream = 0,

@@ -35,7 +35,7 @@ def dispatch_and_check(oracle, cfg_or_shape, topk_np, w_np, x_cpu, scales_cpu, a
     for schedule in gu.SCHEDULES:
         print(f"schedule {schedule}", flush=True)
         recv_x, recv_scales, recv_src_map, h = buf.dispatch(x, scales, topk, w, expert_alignment=align,
-                                                            schedule=schedule)
+                                                            schedule=schedule, zero_pads=True)
         torch.cuda.synchronize()
         buf.status()
         assert h.num_recv_rows() == rows
@@ -135,7 +135,7 @@ def test_scale_factors_through_strides(oracle, schedule):
     buf = ops.Buffer(T, K, E, R, device=gu.DEV)
     recv_x, recv_scales, _, h = buf.dispatch(xq.to(gu.DEV), scales_view, torch.from_numpy(topk_np).to(gu.DEV),
                                              None, expert_alignment=align, column_major_recv_scales=True,
-                                             schedule=schedule)
+                                             schedule=schedule, zero_pads=True)
     torch.cuda.synchronize()
     ref = oracle.full_path(topk_np, None, gu.as_bytes(xq), scales_cpu.numpy(), E, R, align)
     rows = int(ref["expert_offsets"][-1])
@@ -145,9 +145,10 @@ def test_scale_factors_through_strides(oracle, schedule):
     assert (padded[:, T:] == -7.0).all()                                   # the padding was not touched
 
 
-def test_pad_payload_can_be_left_alone(oracle):
-    """With the keep-pad-payload flag the pad rows keep what the buffer held; their map entries
-    and every real row are written as usual."""
+def test_pad_payload_is_left_alone_unless_asked_for_zeros(oracle):
+    """By default the pad rows keep what the buffer held (the reference's receive buffer is not
+    cleared either); their map entries and every real row are written as usual.  With zero_pads the
+    pad rows are zero rows."""
     rng = np.random.default_rng(6)
     T, K, E, R, H, align = 600, 4, 32, 4, 128, 16
     topk_np = wl.uniform_distinct_topk(rng, T, E, K)
@@ -155,9 +156,9 @@ def test_pad_payload_can_be_left_alone(oracle):
     buf = ops.Buffer(T, K, E, R, device=gu.DEV)
     h = buf.dispatch_layout(torch.from_numpy(topk_np).to(gu.DEV), align)
     # same layout handle, once with zero-filled pads and once with the pad payload left alone
-    filled = buf.dispatch(x_cpu.to(gu.DEV), None, torch.from_numpy(topk_np).to(gu.DEV), None, align, handle=h)
-    kept = buf.dispatch(x_cpu.to(gu.DEV), None, torch.from_numpy(topk_np).to(gu.DEV), None, align, handle=h,
-                        zero_pads=False)
+    filled = buf.dispatch(x_cpu.to(gu.DEV), None, torch.from_numpy(topk_np).to(gu.DEV), None, align, handle=h,
+                          zero_pads=True)
+    kept = buf.dispatch(x_cpu.to(gu.DEV), None, torch.from_numpy(topk_np).to(gu.DEV), None, align, handle=h)
     torch.cuda.synchronize()
     ref = oracle.full_path(topk_np, None, gu.as_bytes(x_cpu), None, E, R, align)
     rows = int(ref["expert_offsets"][-1])

@@ -185,7 +185,7 @@ def test_many_pad_rows_under_both_copy_kernels(oracle, zero_pads):
         recv_idx = torch.full((cap,), 77, dtype=torch.int64, device=gu.DEV)
         recv_w = torch.full((cap,), 77.0, dtype=torch.float32, device=gu.DEV)
         slot_map = torch.empty((T, K), dtype=torch.int32, device=gu.DEV)
-        flags = (0 if zero_pads else ops.KEEP_PAD_PAYLOAD) | ops._SCHEDULE_FLAGS[schedule]
+        flags = (ops.ZERO_PAD_PAYLOAD if zero_pads else 0) | ops._SCHEDULE_FLAGS[schedule]
         ops._lib.check(lib.mi_ep_dispatch(
             x_dev.data_ptr(), scales_dev.data_ptr(), topk.data_ptr(), None,
             h.expert_offsets.data_ptr(), h.slot_rel.data_ptr(), h.route_order.data_ptr(),
