@@ -312,9 +312,19 @@ def cpu_baseline(cfg, wk, seconds):
                       f"{threads} OpenMP threads (~{seconds:.0f} s in all)"}
 
 
+def source_fingerprint(path):
+    """sha256 prefix of a C++/HIP source with comments removed and whitespace collapsed: it changes
+    with the code, not with its commentary."""
+    import re
+    text = open(path, encoding="utf-8").read()
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", " ", text)
+    return hashlib.sha256(" ".join(text.split()).encode()).hexdigest()[:16]
+
+
 def measured_traffic(kernel, workload_name):
     """HBM bytes per launch of `kernel` from the committed counter runs, or None when the kernel
-    sources have changed since they were taken (the file records their hashes)."""
+    sources have changed since they were taken (the file records their fingerprints)."""
     path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if not os.path.exists(path):
         return None
@@ -322,7 +332,7 @@ def measured_traffic(kernel, workload_name):
         rec = json.load(f)
     for name, want in rec.get("source_sha16", {}).items():
         src = os.path.join(ROOT, "commbench_amd", "csrc", name)
-        if not os.path.exists(src) or hashlib.sha256(open(src, "rb").read()).hexdigest()[:16] != want:
+        if not os.path.exists(src) or source_fingerprint(src) != want:
             return None
     return rec.get(workload_name, {}).get(kernel)
 

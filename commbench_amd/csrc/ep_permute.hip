@@ -24,7 +24,7 @@
 namespace mi_ep {
 namespace {
 
-constexpr int kPermuteThreads = 256;  // pad-row and pull-mode kernels
+constexpr int kPermuteThreads = 256;  // pull-mode kernels
 constexpr int kPermuteWaves = kPermuteThreads / kWave;
 // The push kernel: small workgroups of two waves and one vector per lane measured best on
 // every row size tried (7, 8 and 14 KiB rows); the kernel is bound by HBM writes, not by
