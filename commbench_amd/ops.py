@@ -104,6 +104,15 @@ class DispatchHandle:
         """Padded row total; synchronises the stream."""
         return int(self.expert_offsets[-1].item())
 
+    def rank_prefix_matrix(self) -> torch.Tensor:
+        """int32[src, dst]: tokens of source chunks 0..src flagged for rank dst, the tokens taken as
+        num_ranks equal contiguous chunks (ceil(T / R) tokens each): the notify example's
+        rank_prefix_matrix (example047 .cu:128-143,352-360) with chunks of this GPU's tokens standing
+        for source ranks.  Needs a layout that ran with num_channels == num_ranks."""
+        _require(self.channel_prefix_matrix is not None and self.channel_prefix_matrix.shape[1] == self.num_ranks,
+                 "rank_prefix_matrix needs a layout with num_channels == num_ranks")
+        return self.channel_prefix_matrix.t().contiguous()
+
 
 class Buffer:
     """Workspace owner, the one-GPU analogue of the reference's ElasticBuffer

@@ -381,18 +381,29 @@ def test_cached_pull_dispatch_and_pull_indices(oracle, payload):
     np.testing.assert_array_equal(pulls.cpu().numpy(), oracle.pull_indices(ref["recv_src_map"], T // 4))
 
 
-def test_rank_prefix_matrix_from_channel_prefix(oracle):
+@pytest.mark.parametrize("shape", [(4096, 8), (4097, 8), (7, 2), (1000, 4), (333, 8), (5, 8)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_rank_prefix_matrix_from_channel_prefix(oracle, shape):
     """One channel per source chunk: channel_prefix_matrix[dst, src] is the notify example's
-    rank_prefix_matrix[src, dst] (example047 .cu:352-360) for R contiguous source chunks."""
-    rng = np.random.default_rng(5)
-    T, K, E, R = 4096, 4, 32, 8
+    rank_prefix_matrix[src, dst] (example047 .cu:352-360) for R contiguous source chunks of
+    ceil(T / R) tokens (its get_channel_task_range, .cu:73-79), ragged and empty chunks included."""
+    T, R = shape
+    print(f"shape {shape}", flush=True)
+    rng = np.random.default_rng(5 + T)
+    K, E = 4, 4 * R
     topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    topk_np[rng.random((T, K)) < 0.3] = -1
     buf = ops.Buffer(T, K, E, R, device=gu.DEV)
     h = buf.dispatch_layout(torch.from_numpy(topk_np).to(gu.DEV), num_channels=R)
     torch.cuda.synchronize()
     _, _, flags = oracle.layout(topk_np, R, E)
-    counts = flags.reshape(R, T // R, R).sum(axis=1).astype(np.int32)
-    np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy().T, oracle.rank_prefix(counts))
+    per_chunk = -(-T // R)
+    counts = np.zeros((R, R), dtype=np.int32)
+    for src in range(R):
+        start = min(per_chunk * src, T)
+        counts[src] = flags[start:min(start + per_chunk, T)].sum(axis=0)
+    np.testing.assert_array_equal(h.rank_prefix_matrix().cpu().numpy(), oracle.rank_prefix(counts))
+    assert (h.rank_prefix_matrix()[-1].cpu().numpy() == h.num_tokens_per_rank.cpu().numpy()).all()
 
 
 def test_combine_ignores_map_entries_beyond_the_rows_it_was_given(oracle):
