@@ -130,3 +130,50 @@ def test_two_streams_with_their_own_workspaces(oracle):
         want = oracle.combine(ref["recv_x"].view(np.uint16), ref["slot_map"], c["w_np"], num_threads=8)
         np.testing.assert_array_equal(gu.bf16_bits(out), want)
         c["buf"].status()
+
+
+def test_host_threads_with_their_own_streams(oracle):
+    """Four host threads, each with its own stream and buffer, launch layout + permute + combine at
+    the same time (ctypes releases the interpreter lock during the calls): the library keeps no
+    mutable state of its own, so every thread must get exactly its own results."""
+    import threading
+    E, R, K, H = 32, 4, 4, 256
+    rng = np.random.default_rng(91)
+    cases = []
+    for i, T in enumerate((900, 1300, 257, 2048)):
+        topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+        w_np = wl.softmax_gates(rng, T, K)
+        x_cpu = wl.bf16_normal(rng, T, H)
+        cases.append(dict(T=T, topk_np=topk_np, w_np=w_np, x_cpu=x_cpu, buf=ops.Buffer(T, K, E, R, device=gu.DEV),
+                          topk=torch.from_numpy(topk_np).to(gu.DEV), w=torch.from_numpy(w_np).to(gu.DEV),
+                          x=x_cpu.to(gu.DEV), stream=torch.cuda.Stream(), schedule=gu.SCHEDULES[i % 2]))
+    torch.cuda.synchronize()
+    results, errors = [None] * len(cases), []
+
+    def work(i):
+        c = cases[i]
+        try:
+            with torch.cuda.stream(c["stream"]):
+                for _ in range(10):
+                    recv_x, _, _, h = c["buf"].dispatch(c["x"], None, c["topk"], c["w"], schedule=c["schedule"])
+                    out = ops.combine(recv_x, h, c["w"])
+                c["stream"].synchronize()
+            results[i] = (recv_x, h, out)
+        except Exception as exc:          # reported by the main thread
+            errors.append((i, repr(exc)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(cases))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for c, (recv_x, h, out) in zip(cases, results):
+        ref = oracle.full_path(c["topk_np"], c["w_np"], gu.as_bytes(c["x_cpu"]), None, E, R)
+        rows = int(ref["expert_offsets"][-1])
+        np.testing.assert_array_equal(h.slot_map.cpu().numpy(), ref["slot_map"])
+        np.testing.assert_array_equal(gu.as_bytes(recv_x)[:rows], ref["recv_x"])
+        want = oracle.combine(ref["recv_x"].view(np.uint16), ref["slot_map"], c["w_np"], num_threads=8)
+        np.testing.assert_array_equal(gu.bf16_bits(out), want)
+        c["buf"].status()
