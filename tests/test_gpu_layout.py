@@ -176,3 +176,22 @@ def test_expired_wait_terminates_and_is_reported(oracle):
                                         torch.cuda.current_stream().cuda_stream), "re-init")
     _, h = gu.run_fused_layout(buf, topk_np)
     gu.check_layout_against_oracle(oracle, h, topk_np, R, E)
+
+
+@pytest.mark.parametrize("tokens", [3000, 20000], ids=["static_tiles", "tiles_by_arrival"])
+def test_generation_counter_wraps_around(oracle, tokens):
+    """The look-back's status words are told apart by a 30-bit generation in the workspace's turn
+    word.  Starting two launches before the counter's end, five launches in a row (the last three
+    after the wrap) must all see only their own words."""
+    E, R, K = 64, 8, 4
+    rng = np.random.default_rng(tokens)
+    buf = ops.Buffer(tokens, K, E, R, device=gu.DEV)
+    torch.cuda.synchronize()
+    turn = buf.workspace[:8].view(torch.int64)
+    turn[0] = (0x3FFFFFFF - 1) << 32          # {generation = 2^30 - 2, arrivals = 0}
+    for launch in range(5):
+        T = tokens - 17 * launch
+        topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+        _, h = gu.run_fused_layout(buf, topk_np, expert_alignment=3, num_channels=8)
+        gu.check_layout_against_oracle(oracle, h, topk_np, R, E, align=3, channels=8)
+    assert int(turn[0].item()) >> 32 == 3       # 2^30 - 2 + 5 launches, modulo 2^30
