@@ -139,10 +139,16 @@ __global__ __launch_bounds__(kCombineThreads) void ep_combine_kernel(const Combi
   }
 }
 
-template <int kTopk>
+// Persistent schedule.  A group is `group_tokens` consecutive tokens of one workgroup; its units
+// (token, KiB batch), numbered row by row, are staged before one burst writes them out: units below
+// `lds_units` in LDS (1 KiB slot per unit), the following 16 * kRegUnits in registers of the wave
+// that computed them (unit lds_units + 16 r + w is register r of wave w).  The register tail makes
+// groups longer than the LDS alone allows; it is used where that turns two bursts into one.
+template <int kTopk, int kRegUnits>
 __global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const CombineArgs a,
-                                                                          const int group_tokens) {
-  extern __shared__ vec16 stage[];  // [group_tokens][row_vecs]
+                                                                          const int group_tokens,
+                                                                          const int lds_units) {
+  extern __shared__ vec16 stage[];  // [lds_units][64]
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
   const int batches = (a.row_vecs + kWave - 1) / kWave;
@@ -154,23 +160,62 @@ __global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const
     const int g0 = g * group_tokens;
     const int gn = a.num_tokens - g0 < group_tokens ? a.num_tokens - g0 : group_tokens;
     const int units = gn * batches;
-    for (int u = wave; u < units; u += kStagedWaves) {
-      const int local = u / batches;
-      const int batch = u - local * batches;
-      vec16 out[1];
-      combine_unit<kTopk, 1>(a, g0 + local, batch, lane, out);
-      const int v = batch * kWave + lane;
-      if (v < a.row_vecs) stage[local * a.row_vecs + v] = out[0];
+    const int in_lds = units < lds_units ? units : lds_units;
+    {
+      // unit u = wave, wave + 16, ...: (local, batch) stepped along instead of divided out
+      int local = wave / batches, batch = wave - local * batches;
+      for (int u = wave; u < in_lds; u += kStagedWaves) {
+        vec16 out[1];
+        combine_unit<kTopk, 1>(a, g0 + local, batch, lane, out);
+        stage[u * kWave + lane] = out[0];
+        batch += kStagedWaves;
+        while (batch >= batches) {
+          batch -= batches;
+          ++local;
+        }
+      }
+    }
+    vec16 keep[kRegUnits > 0 ? kRegUnits : 1];
+#pragma unroll
+    for (int r = 0; r < kRegUnits; ++r) {
+      const int u = lds_units + r * kStagedWaves + wave;
+      if (u < units) {  // wave-uniform
+        const int local = u / batches;
+        vec16 out[1];
+        combine_unit<kTopk, 1>(a, g0 + local, u - local * batches, lane, out);
+        keep[r] = out[0];
+      }
     }
     __syncthreads();
-    // The group's rows are contiguous in combined_x: one linear burst.
+    // The group's rows are contiguous in combined_x: one burst, first what the LDS holds (every
+    // thread takes 16-byte pieces in order), then each wave's own registers.
     vec16* dst = a.combined_x + static_cast<size_t>(g0) * a.row_vecs;
-    const int n = gn * a.row_vecs;
-    for (int i = static_cast<int>(threadIdx.x); i < n; i += kStagedThreads)
-      __builtin_nontemporal_store(stage[i], dst + i);
+    {
+      int local = wave / batches, batch = wave - local * batches;
+      for (int u = wave; u < in_lds; u += kStagedWaves) {
+        const int v = batch * kWave + lane;
+        if (v < a.row_vecs) __builtin_nontemporal_store(stage[u * kWave + lane], dst + local * a.row_vecs + v);
+        batch += kStagedWaves;
+        while (batch >= batches) {
+          batch -= batches;
+          ++local;
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kRegUnits; ++r) {
+      const int u = lds_units + r * kStagedWaves + wave;
+      if (u < units) {
+        const int local = u / batches;
+        const int v = (u - local * batches) * kWave + lane;
+        if (v < a.row_vecs) __builtin_nontemporal_store(keep[r], dst + local * a.row_vecs + v);
+      }
+    }
     __syncthreads();
   }
 }
+
+constexpr int kStagedRegUnits = 4;  // units per wave kept in registers when that makes one burst do
 
 template <int kTopk>
 hipError_t launch_combine_k(const CombineArgs& a, hipStream_t stream) {
@@ -184,28 +229,46 @@ hipError_t launch_combine_k(const CombineArgs& a, hipStream_t stream) {
   // Large shapes: persistent staged schedule.  It needs enough tokens per CU for
   // its phases to be long, and rows that fit the staging area.
   if (a.num_tokens >= 16 * cus && row_bytes >= 2048 && row_bytes <= kStageBytes) {
-    // Phases of equal length on every CU: split a CU's share of the tokens into the
-    // fewest groups that fit the staging area.
+    // Phases of equal length on every CU: split a CU's share of the tokens into the fewest groups
+    // that fit the staging area, with the register tail only if it makes a single burst possible.
+    const int batches = (a.row_vecs + kWave - 1) / kWave;
     const int tokens_per_wg = (a.num_tokens + cus - 1) / cus;
-    const int max_group = static_cast<int>(kStageBytes / row_bytes);
-    const int phases = (tokens_per_wg + max_group - 1) / max_group;
+    const int lds_capacity = static_cast<int>(kStageBytes / (kWave * sizeof(vec16)));  // units of 1 KiB
+    const int rows_lds = lds_capacity / batches;
+    const int rows_reg = (lds_capacity + kStagedRegUnits * kStagedWaves) / batches;
+    const int phases_lds = (tokens_per_wg + rows_lds - 1) / rows_lds;
+    const int phases_reg = (tokens_per_wg + rows_reg - 1) / rows_reg;
+    // Measured: going from two bursts to one is worth 1-3 us (4096 x 14 KiB rows: 85 -> 82 us);
+    // three to two gains nothing at 8192 rows and four to three loses 3 us at 16384 x 8 KiB, where
+    // the unrolled tail's registers and code cost more than the boundary it saves.
+    const bool with_registers = phases_reg == 1 && phases_lds > 1;
+    const int phases = with_registers ? phases_reg : phases_lds;
     const int group_tokens = (tokens_per_wg + phases - 1) / phases;
+    const int group_units = group_tokens * batches;
+    const int lds_units = group_units < lds_capacity ? group_units : lds_capacity;
     const int groups = (a.num_tokens + group_tokens - 1) / group_tokens;
     const int grid = groups < cus ? groups : cus;
-    const size_t lds = static_cast<size_t>(group_tokens) * row_bytes;
+    const size_t lds = static_cast<size_t>(lds_units) * kWave * sizeof(vec16);
     // The kernel's LDS ceiling is raised once per device (a function attribute lives with the
-    // device's copy of the code object); the flag only ever goes from 0 to 1.
+    // device's copy of the code object); the flags only ever go from 0 to 1.
     constexpr int kMaxDevices = 64;
-    static std::atomic<int> lds_limit_raised[kMaxDevices];
+    static std::atomic<int> lds_limit_raised[2][kMaxDevices];
     if (ordinal < 0 || ordinal >= kMaxDevices) return hipErrorInvalidDevice;
-    if (lds_limit_raised[ordinal].load(std::memory_order_acquire) == 0) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ep_combine_staged_kernel<kTopk>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes);
+    const void* kernel = with_registers
+                             ? reinterpret_cast<const void*>(&ep_combine_staged_kernel<kTopk, kStagedRegUnits>)
+                             : reinterpret_cast<const void*>(&ep_combine_staged_kernel<kTopk, 0>);
+    std::atomic<int>& raised = lds_limit_raised[with_registers ? 1 : 0][ordinal];
+    if (raised.load(std::memory_order_acquire) == 0) {
+      const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes);
       if (e != hipSuccess) return e;
-      lds_limit_raised[ordinal].store(1, std::memory_order_release);
+      raised.store(1, std::memory_order_release);
     }
-    hipLaunchKernelGGL((ep_combine_staged_kernel<kTopk>), dim3(grid), dim3(kStagedThreads), lds, stream, a,
-                       group_tokens);
+    if (with_registers)
+      hipLaunchKernelGGL((ep_combine_staged_kernel<kTopk, kStagedRegUnits>), dim3(grid), dim3(kStagedThreads), lds,
+                         stream, a, group_tokens, lds_units);
+    else
+      hipLaunchKernelGGL((ep_combine_staged_kernel<kTopk, 0>), dim3(grid), dim3(kStagedThreads), lds, stream, a,
+                         group_tokens, lds_units);
     return hipGetLastError();
   }
   // Everything else: one unit per wave; two vectors per lane once rows are long.

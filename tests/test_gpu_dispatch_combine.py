@@ -259,11 +259,14 @@ def test_combine_every_topk_with_biases(oracle, K):
         assert worst == 0, "same fma chain on both sides: expected bit-exact"
 
 
-@pytest.mark.parametrize("shape", [(4099, 3, 1032), (6000, 8, 2048), (4096, 1, 1024), (9001, 5, 1280)],
+@pytest.mark.parametrize("shape", [(4099, 3, 1032), (6000, 8, 2048), (4096, 1, 1024), (9001, 5, 1280),
+                                   (4099, 2, 5000), (5000, 8, 4232), (4100, 4, 7168)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_combine_large_token_counts_use_the_staged_schedule(oracle, shape):
     """>= 16 tokens per compute unit and rows >= 2 KiB take the persistent LDS-staged schedule:
-    ragged token ranges, ragged last vectors, masks, weights on/off and both biases."""
+    ragged token ranges, ragged last vectors, masks, weights on/off and both biases.  The last three
+    shapes need more staging than the LDS holds for a single burst (170, 180 and 238 KiB per
+    workgroup): the first two put the rest in registers, the third takes two bursts."""
     T, K, H = shape
     print(f"shape {shape}", flush=True)
     rng = np.random.default_rng(T + K)
