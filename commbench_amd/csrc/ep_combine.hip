@@ -32,6 +32,14 @@ constexpr int kCombineWaves = kCombineThreads / kWave;
 constexpr int kStagedThreads = 1024;
 constexpr int kStagedWaves = kStagedThreads / kWave;
 constexpr int kStageBytes = 160 * 1024;  // all of the CU's LDS: one workgroup per CU
+// Raw buffer descriptor word 3 for 32-bit elements on this architecture, and the cache-policy
+// operand of buffer instructions (bit 1: streaming hint "nt"; bit 4: device scope "sc1").
+constexpr int kRawBufferFormat = 0x00020000;
+constexpr int kCachePolicyStreaming = 2;
+constexpr int kCachePolicyDeviceScope = 16;
+// Outputs that leave room in the memory-side cache (256 MB on this part; not reported by the
+// runtime) for an input of their own size are written through into it: a little under half of it.
+constexpr long long kStoreThroughBytesMax = 120ll * 1024 * 1024;
 
 // Computes one unit; out[u] holds the packed bf16 of vector v0 + u * 64 (valid
 // where that index is inside the row).
@@ -144,10 +152,20 @@ __global__ __launch_bounds__(kCombineThreads) void ep_combine_kernel(const Combi
 // `lds_units` in LDS (1 KiB slot per unit), the following 16 * kRegUnits in registers of the wave
 // that computed them (unit lds_units + 16 r + w is register r of wave w).  The register tail makes
 // groups longer than the LDS alone allows; it is used where that turns two bursts into one.
+//
+// The burst's stores come in two kinds.  Written through at device scope ("sc1", no streaming hint)
+// they are taken up by the 256 MB memory-side cache and reach HBM later, largely while the next,
+// latency-bound kernel leaves it idle: the kernel no longer pays for turning the memory bus around
+// in the middle of its reads (8192 x 14 KiB rows: 174 -> 164 us, whole step 346 -> 338 us).  That
+// holds while the output and an input of its size that the next step re-reads both fit that cache;
+// beyond, the dirty lines fall out during the next kernel's writes and cost it more than was gained
+// (176 MB of output: this kernel -12 us, the following copy +32 us), so larger outputs are streamed
+// ("nt") as before.
 template <int kTopk, int kRegUnits>
 __global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const CombineArgs a,
                                                                           const int group_tokens,
-                                                                          const int lds_units) {
+                                                                          const int lds_units,
+                                                                          const int store_through) {
   extern __shared__ vec16 stage[];  // [lds_units][64]
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
@@ -190,11 +208,22 @@ __global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const
     // The group's rows are contiguous in combined_x: one burst, first what the LDS holds (every
     // thread takes 16-byte pieces in order), then each wave's own registers.
     vec16* dst = a.combined_x + static_cast<size_t>(g0) * a.row_vecs;
+    // A buffer descriptor over the group's rows: the store's cache policy is an operand of the buffer
+    // form of the instruction (and stores beyond the descriptor's end would be dropped).
+    const __amdgpu_buffer_rsrc_t group_rows =
+        __builtin_amdgcn_make_buffer_rsrc(dst, 0, gn * a.row_vecs * static_cast<int>(sizeof(vec16)), kRawBufferFormat);
+    auto store = [&](const vec16 value, const int vec_index) {
+      const int offset = vec_index * static_cast<int>(sizeof(vec16));
+      if (store_through)
+        __builtin_amdgcn_raw_buffer_store_b128(value, group_rows, offset, 0, kCachePolicyDeviceScope);
+      else
+        __builtin_amdgcn_raw_buffer_store_b128(value, group_rows, offset, 0, kCachePolicyStreaming);
+    };
     {
       int local = wave / batches, batch = wave - local * batches;
       for (int u = wave; u < in_lds; u += kStagedWaves) {
         const int v = batch * kWave + lane;
-        if (v < a.row_vecs) __builtin_nontemporal_store(stage[u * kWave + lane], dst + local * a.row_vecs + v);
+        if (v < a.row_vecs) store(stage[u * kWave + lane], local * a.row_vecs + v);
         batch += kStagedWaves;
         while (batch >= batches) {
           batch -= batches;
@@ -208,7 +237,7 @@ __global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const
       if (u < units) {
         const int local = u / batches;
         const int v = (u - local * batches) * kWave + lane;
-        if (v < a.row_vecs) __builtin_nontemporal_store(keep[r], dst + local * a.row_vecs + v);
+        if (v < a.row_vecs) store(keep[r], local * a.row_vecs + v);
       }
     }
     __syncthreads();
@@ -263,12 +292,13 @@ hipError_t launch_combine_k(const CombineArgs& a, hipStream_t stream) {
       if (e != hipSuccess) return e;
       raised.store(1, std::memory_order_release);
     }
+    const int store_through = static_cast<long long>(a.num_tokens) * row_bytes <= kStoreThroughBytesMax ? 1 : 0;
     if (with_registers)
       hipLaunchKernelGGL((ep_combine_staged_kernel<kTopk, kStagedRegUnits>), dim3(grid), dim3(kStagedThreads), lds,
-                         stream, a, group_tokens, lds_units);
+                         stream, a, group_tokens, lds_units, store_through);
     else
       hipLaunchKernelGGL((ep_combine_staged_kernel<kTopk, 0>), dim3(grid), dim3(kStagedThreads), lds, stream, a,
-                         group_tokens, lds_units);
+                         group_tokens, lds_units, store_through);
     return hipGetLastError();
   }
   // Everything else: one unit per wave; two vectors per lane once rows are long.
