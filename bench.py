@@ -22,6 +22,7 @@ if ROOT not in sys.path:
 
 PEAK_HBM_GBPS = 8000.0      # MI355X published HBM3E bandwidth
 ZERO_PAD_PAYLOAD = 1        # MI_EP_DISPATCH_ZERO_PAD_PAYLOAD
+STREAM_OUTPUT = 1           # MI_EP_COMBINE_STREAM_OUTPUT
 
 
 def parse_args():
@@ -117,6 +118,8 @@ class Workload:
         self.recv_idx = torch.empty(cap, dtype=torch.int64, device=dev)
         self.recv_w = torch.empty(cap, dtype=torch.float32, device=dev)
         self.out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+        self.out_ring = [self.out]
+        self.combine_flags = 0
         ws_bytes = self.lib.mi_ep_workspace_bytes(T, K, E, R)
         self.ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         self.stream = torch.cuda.current_stream().cuda_stream
@@ -155,9 +158,10 @@ class Workload:
 
     def combine(self):
         c = self.cfg
+        out = self.out_ring[self.step_index % len(self.out_ring)]
         self._lib.check(self.lib.mi_ep_combine(
             self.y.data_ptr(), self.cap, self.slot_map.data_ptr(), self.w.data_ptr(), None, None, None, None,
-            c.num_tokens, c.num_topk, c.hidden, self.out.data_ptr(), None, None, self.stream), "combine")
+            c.num_tokens, c.num_topk, c.hidden, out.data_ptr(), None, None, self.combine_flags, self.stream), "combine")
 
     def step(self):
         self.layout()
@@ -230,7 +234,7 @@ class RankWorkload:
         c = self.cfg
         self._lib.check(self.lib.mi_ep_combine(
             self.y.data_ptr(), self.cap, self.combine_map.data_ptr(), None, None, None, None, None,
-            c.num_tokens, c.num_topk, c.hidden, self.out.data_ptr(), None, None, self.stream), "combine")
+            c.num_tokens, c.num_topk, c.hidden, self.out.data_ptr(), None, None, 0, self.stream), "combine")
 
     def step(self):
         self.layout()
@@ -428,19 +432,34 @@ def main():
 
     # The same steps with the source rows cycling through three buffers, so that they come from
     # HBM instead of the 256 MB memory-side cache that keeps a single re-read source resident.
-    cold_ms_per_step = None
+    # Then also with the combined output cycling through three buffers: the combine writes outputs
+    # of up to 120 MiB through into the memory-side cache, and an output buffer that is rewritten every
+    # step would never have to leave it; three of them do.
+    # That case is measured under both output policies of the combine: written through (the default)
+    # and streamed straight to HBM (MI_EP_COMBINE_STREAM_OUTPUT).
+    cold_ms_per_step = cold_both_ms_per_step = cold_both_streamed_ms_per_step = None
     if len(wk.x_ring) == 1 and not args.no_cold_source:
         ring = wk.x_ring
         wk.x_ring = [wk.x, wk.x.clone(), wk.x.clone()]
-        for _ in range(6):
-            wk.step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            wk.step()
-        torch.cuda.synchronize()
-        cold_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+        def cold_pass():
+            for _ in range(9):
+                wk.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                wk.step()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3 / args.steps
+
+        cold_ms_per_step = cold_pass()
+        wk.out_ring = [wk.out, torch.empty_like(wk.out), torch.empty_like(wk.out)]
+        cold_both_ms_per_step = cold_pass()
+        wk.combine_flags = STREAM_OUTPUT
+        cold_both_streamed_ms_per_step = cold_pass()
+        wk.combine_flags = 0
         wk.x_ring = ring
+        wk.out_ring = [wk.out]
         wk.step()
         torch.cuda.synchronize()
 
@@ -565,6 +584,16 @@ def main():
             "tokens_per_s": T / (cold_ms_per_step * 1e-3),
             "hbm_frac_whole_step": wk.bytes["total"] / (cold_ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
             "note": "source rows cycled through 3 buffers so that they are read from HBM"},
+        "cold_source_and_sink": None if cold_both_ms_per_step is None else {
+            "ms_per_step": cold_both_ms_per_step,
+            "tokens_per_s": T / (cold_both_ms_per_step * 1e-3),
+            "hbm_frac_whole_step": wk.bytes["total"] / (cold_both_ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+            "streamed_output_ms_per_step": cold_both_streamed_ms_per_step,
+            "streamed_output_hbm_frac_whole_step": wk.bytes["total"] / (cold_both_streamed_ms_per_step * 1e-3) / 1e9
+                                                   / PEAK_HBM_GBPS,
+            "note": "source rows and combined output each cycled through 3 buffers: every counted byte "
+                    "crosses the HBM interface; once with the combine's output written through the "
+                    "memory-side cache (default), once streamed to HBM (MI_EP_COMBINE_STREAM_OUTPUT)"},
         "algorithmic_bytes": wk.bytes,
         "device_traits": traits,
         "kernel_us": kernel_us,

@@ -43,7 +43,7 @@ SIGNATURES = {
     "mi_ep_combine_rank_weights": (_int, [_vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp]),
     "mi_ep_dispatch_cached": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _int, _vp]),
     "mi_ep_pull_indices": (_int, [_vp, _int, _int, _vp, _vp]),
-    "mi_ep_combine": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp, _vp]),
+    "mi_ep_combine": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp, _int, _vp]),
     "mi_ep_host_get_dispatch_layout": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int]),
     "mi_ep_host_dispatch_layout": (_int, [_vp, _int, _int, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp,
                                           _vp, _vp, _int, _vp, _vp, _vp, _vp]),

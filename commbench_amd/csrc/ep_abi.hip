@@ -484,8 +484,9 @@ int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float*
                   const void* bias_0, const void* bias_1, const float* recv_topk_weights,
                   const int64_t* recv_topk_idx, int num_tokens, int num_topk, int hidden,
                   void* combined_x, float* combined_topk_weights, int64_t* combined_topk_idx,
-                  void* stream) {
+                  int flags, void* stream) {
   if (!route_count_ok(num_tokens, num_topk)) return MI_EP_EINVAL;
+  if ((flags & ~MI_EP_COMBINE_STREAM_OUTPUT) != 0) return MI_EP_EINVAL;
   if (hidden <= 0 || hidden % 8 != 0 || num_rows < 0) return MI_EP_EINVAL;
   // Units of the staged schedule are counted in int: rows of a group times 16-byte vectors.
   if (static_cast<long long>(hidden) / 8 >= (1LL << 24)) return MI_EP_EINVAL;
@@ -511,6 +512,7 @@ int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float*
   a.num_topk = num_topk;
   a.num_rows = num_rows;
   a.row_vecs = hidden / 8;
+  a.stream_output = (flags & MI_EP_COMBINE_STREAM_OUTPUT) != 0 ? 1 : 0;
   return status_of(launch_combine(a, as_stream(stream)));
 }
 

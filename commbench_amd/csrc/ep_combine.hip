@@ -292,7 +292,8 @@ hipError_t launch_combine_k(const CombineArgs& a, hipStream_t stream) {
       if (e != hipSuccess) return e;
       raised.store(1, std::memory_order_release);
     }
-    const int store_through = static_cast<long long>(a.num_tokens) * row_bytes <= kStoreThroughBytesMax ? 1 : 0;
+    const int store_through =
+        (!a.stream_output && static_cast<long long>(a.num_tokens) * row_bytes <= kStoreThroughBytesMax) ? 1 : 0;
     if (with_registers)
       hipLaunchKernelGGL((ep_combine_staged_kernel<kTopk, kStagedRegUnits>), dim3(grid), dim3(kStagedThreads), lds,
                          stream, a, group_tokens, lds_units, store_through);

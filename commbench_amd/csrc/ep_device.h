@@ -178,6 +178,7 @@ struct CombineArgs {
   int num_topk;
   int num_rows;  // rows of y; map entries at or beyond it are treated as non-routes
   int row_vecs;  // 16-byte vectors (8 bf16) per row
+  int stream_output;  // 1: combined_x goes straight to HBM whatever its size
 };
 
 hipError_t launch_combine(const CombineArgs& a, hipStream_t stream);

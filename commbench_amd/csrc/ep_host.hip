@@ -340,7 +340,7 @@ int mi_ep_host_combine(const void* y, int num_rows, const int* slot_map, const f
   uint16_t* d_out = s.alloc<uint16_t>(th);
   if (!s.ok()) return s.status(MI_EP_OK);
   int code = mi_ep_combine(d_y, num_rows, d_map, d_w, d_b0, d_b1, nullptr, nullptr, num_tokens, num_topk,
-                           hidden, d_out, nullptr, nullptr, nullptr);
+                           hidden, d_out, nullptr, nullptr, MI_EP_COMBINE_STREAM_OUTPUT, nullptr);  // read back over PCIe next
   code = sync_status(code);
   if (code != MI_EP_OK) return code;
   s.download(static_cast<uint16_t*>(combined_x), d_out, th);

@@ -33,6 +33,7 @@ MAX_EXPERTS = 1024
 ZERO_PAD_PAYLOAD = 1   # MI_EP_DISPATCH_ZERO_PAD_PAYLOAD
 BY_TOKEN = 2           # MI_EP_DISPATCH_BY_TOKEN
 BY_DESTINATION = 4     # MI_EP_DISPATCH_BY_DESTINATION
+STREAM_OUTPUT = 1      # MI_EP_COMBINE_STREAM_OUTPUT
 _SCHEDULE_FLAGS = {"auto": 0, "token": BY_TOKEN, "destination": BY_DESTINATION}
 
 
@@ -372,13 +373,15 @@ def combine(y: torch.Tensor, slot_map: Union[torch.Tensor, DispatchHandle],
             topk_weights: Optional[torch.Tensor] = None,
             bias: Union[None, torch.Tensor, Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]] = None,
             recv_topk_weights: Optional[torch.Tensor] = None,
-            recv_topk_idx: Optional[torch.Tensor] = None):
+            recv_topk_idx: Optional[torch.Tensor] = None, stream_output: bool = False):
     """combined_x[t] = bf16(sum_k w[t,k] * y[slot_map[t,k]] (+ biases)), fp32 accumulation.
 
     topk_weights=None gives the reference's plain ordered sum.  When `recv_topk_weights` (the
     per-row weights that travelled with dispatch) is given, also returns them gathered back to
     [num_tokens, num_topk], as the reference's combined_topk_weights; `recv_topk_idx` (the per-row
     expert ids) likewise comes back as combined_topk_idx, after the weights.
+    `stream_output` sends the result straight to HBM instead of through the memory-side cache
+    (MI_EP_COMBINE_STREAM_OUTPUT): for outputs that nothing reads soon.
     """
     if isinstance(slot_map, DispatchHandle):
         _require(slot_map.slot_map is not None, "handle has not been through dispatch")
@@ -416,7 +419,8 @@ def combine(y: torch.Tensor, slot_map: Union[torch.Tensor, DispatchHandle],
     lib = _lib.load()
     _lib.check(lib.mi_ep_combine(_ptr(y), y.shape[0], _ptr(slot_map), _ptr(topk_weights), _ptr(bias_0),
                                  _ptr(bias_1), _ptr(recv_topk_weights), _ptr(recv_topk_idx), T, K, H,
-                                 _ptr(out), _ptr(out_w), _ptr(out_i), _stream()), "mi_ep_combine")
+                                 _ptr(out), _ptr(out_w), _ptr(out_i), STREAM_OUTPUT if stream_output else 0,
+                                 _stream()), "mi_ep_combine")
     if out_w is None and out_i is None:
         return out
     return tuple(t for t in (out, out_w, out_i) if t is not None)

@@ -342,12 +342,21 @@ int mi_ep_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_sou
  *   recv_topk_idx / combined_topk_idx   both NULL, or int64[rows] in and
  *                int64[num_tokens, num_topk] out: the expert ids that travelled with the rows
  *                (-1 for non-routes; combined_topk_idx, example083 .cu:26)
+ *   flags        0, or MI_EP_COMBINE_STREAM_OUTPUT.  By default an output of up to 120 MiB is
+ *                written through into the GPU's memory-side cache (256 MB), where the operator
+ *                that consumes it next finds it and from where it reaches HBM later; the kernel
+ *                itself is then almost a pure read stream (about 5 % faster on large shapes).
+ *                With the flag, and always beyond 120 MiB, the output is streamed straight to
+ *                HBM: the choice for an output that nothing reads soon, since lines that fall
+ *                out of that cache during other memory-bound kernels cost those more than the
+ *                flag costs this one.  The results are identical.
  */
+#define MI_EP_COMBINE_STREAM_OUTPUT 1
 int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
                   const void* bias_0, const void* bias_1, const float* recv_topk_weights,
                   const int64_t* recv_topk_idx, int num_tokens, int num_topk, int hidden,
                   void* combined_x, float* combined_topk_weights, int64_t* combined_topk_idx,
-                  void* stream);
+                  int flags, void* stream);
 
 /*
  * Host-pointer twins: the same operations with every pointer in ordinary host memory.  Each call

@@ -222,7 +222,7 @@ class ExpertParallelBuffer {
   void combine_ranks(const void* d_y, int num_rows, const void* d_bias_0, const void* d_bias_1, int hidden,
                      void* d_combined_x, hipStream_t stream = 0) const {
     MI_EP_CHECK(mi_ep_combine(d_y, num_rows, h_.rank_combine_map, nullptr, d_bias_0, d_bias_1, nullptr, nullptr,
-                              h_.num_tokens, num_topk_, hidden, d_combined_x, nullptr, nullptr, stream));
+                              h_.num_tokens, num_topk_, hidden, d_combined_x, nullptr, nullptr, /*flags=*/0, stream));
   }
 
   // combined_x[t] = bf16(sum_k w[t,k] * y[slot_map[t,k]] + bias_0 + bias_1); null weights = plain sum.
@@ -237,7 +237,7 @@ class ExpertParallelBuffer {
                               d_combined_topk_weights != nullptr ? h_.recv_topk_weights : nullptr,
                               d_combined_topk_idx != nullptr ? h_.recv_topk_idx : nullptr, h_.num_tokens,
                               num_topk_, hidden, d_combined_x, d_combined_topk_weights, d_combined_topk_idx,
-                              stream));
+                              /*flags=*/0, stream));
   }
 
   // Synchronises the stream; exits if a device-side bounded wait ever expired.

@@ -123,9 +123,11 @@ def test_host_only_entry_points():
     assert lib.mi_ep_dispatch_layout_static(None, 1 << 20, 2, 8, 1024, 1, 0, None, None, None, None, None, None,
                                             None, None, 0, None, None, None, None, None, None) == -7   # beyond the scratch
     assert lib.mi_ep_workspace_set_wait_limit(None, 1, None) == -22
-    assert lib.mi_ep_combine(None, 0, None, None, None, None, None, None, 4, 2, 12, None, None, None, None) == -22
+    assert lib.mi_ep_combine(None, 0, None, None, None, None, None, None, 4, 2, 12, None, None, None, 0, None) == -22
     assert lib.mi_ep_combine(None, 0, None, None, None, None, None, None, 1 << 28, 8, 16, None, None, None,
-                             None) == -22                                              # T * K beyond 2^30
+                             0, None) == -22                                           # T * K beyond 2^30
+    assert lib.mi_ep_combine(None, 0, None, None, None, None, None, None, 0, 2, 16, None, None, None,
+                             2, None) == -22                                           # unknown flag
     assert lib.mi_ep_dispatch(None, None, None, None, None, None, None, None, 4, 2, 8, 1, 24, 0,
                               None, None, None, None, None, None, 0, 0, None) == -22   # 24 % 16 != 0
 

@@ -55,7 +55,7 @@ def test_graph_replays_match_eager(oracle, schedule):
             recv_idx.data_ptr(), recv_w.data_ptr(), slot_map.data_ptr(), cap, schedule, stream), "dispatch")
         _lib.check(lib.mi_ep_combine(
             recv_x.data_ptr(), cap, slot_map.data_ptr(), w.data_ptr(), None, None, None, None, T, K, H,
-            out.data_ptr(), None, None, stream), "combine")
+            out.data_ptr(), None, None, 0, stream), "combine")
 
     def load_inputs(seed):
         r = np.random.default_rng(seed)
