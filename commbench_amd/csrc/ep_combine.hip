@@ -68,19 +68,22 @@ __device__ __forceinline__ void combine_unit(const CombineArgs& a, const int tok
     for (int i = 0; i < 8; ++i) acc[u][i] = 0.0f;
 
   if (routed != 0) {
-    // Non-routes load the token's first routed row again (a cache hit) so that
-    // every load can be issued before the first multiply-add.
-    const int fallback = wave_read(slot, __builtin_ctzll(routed));
+    // Every load is issued before the first multiply-add, as straight-line code: each row is read
+    // through a buffer descriptor of its own, one row long for a route and empty for a non-route, so
+    // that lanes past the row's end and the loads of non-routes are dropped by the bounds check (they
+    // return zeros without a memory request) instead of being branched around.
     vec16 buf[kTopk][kBatchVecs];
+    const int row_bytes = a.row_vecs * static_cast<int>(sizeof(vec16));
 #pragma unroll
     for (int k = 0; k < kTopk; ++k) {
       const int row = wave_read(slot, k);
-      const vec16* src = a.y + static_cast<size_t>(row >= 0 ? row : fallback) * a.row_vecs;
+      const __amdgpu_buffer_rsrc_t row_k = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<vec16*>(a.y + static_cast<size_t>(row >= 0 ? row : 0) * a.row_vecs), 0,
+          row >= 0 ? row_bytes : 0, kRawBufferFormat);
 #pragma unroll
-      for (int u = 0; u < kBatchVecs; ++u) {
-        const int v = v0 + u * kWave;
-        if (v < a.row_vecs) buf[k][u] = __builtin_nontemporal_load(src + v);
-      }
+      for (int u = 0; u < kBatchVecs; ++u)
+        buf[k][u] = __builtin_amdgcn_raw_buffer_load_b128(row_k, (v0 + u * kWave) * static_cast<int>(sizeof(vec16)), 0,
+                                                          kCachePolicyStreaming);
     }
 #pragma unroll
     for (int k = 0; k < kTopk; ++k) {
