@@ -32,11 +32,6 @@ constexpr int kCombineWaves = kCombineThreads / kWave;
 constexpr int kStagedThreads = 1024;
 constexpr int kStagedWaves = kStagedThreads / kWave;
 constexpr int kStageBytes = 160 * 1024;  // all of the CU's LDS: one workgroup per CU
-// Raw buffer descriptor word 3 for 32-bit elements on this architecture, and the cache-policy
-// operand of buffer instructions (bit 1: streaming hint "nt"; bit 4: device scope "sc1").
-constexpr int kRawBufferFormat = 0x00020000;
-constexpr int kCachePolicyStreaming = 2;
-constexpr int kCachePolicyDeviceScope = 16;
 // Outputs that leave room in the memory-side cache (256 MB on this part; not reported by the
 // runtime) for an input of their own size are written through into it: a little under half of it.
 constexpr long long kStoreThroughBytesMax = 120ll * 1024 * 1024;

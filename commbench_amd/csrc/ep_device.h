@@ -11,6 +11,11 @@ namespace mi_ep {
 typedef uint32_t vec16 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
+// Raw buffer descriptor word 3 for 32-bit elements on this architecture, and the cache-policy
+// operand of buffer instructions (bit 1: streaming hint "nt"; bit 4: device scope "sc1").
+constexpr int kRawBufferFormat = 0x00020000;
+constexpr int kCachePolicyStreaming = 2;
+constexpr int kCachePolicyDeviceScope = 16;
 constexpr int kMaxRanks = 8;
 constexpr int kMaxTopk = 8;
 constexpr int kMaxExperts = 1024;

@@ -11,10 +11,13 @@
 //
 // Shape of the computation (wave64):
 //   * a tile is 256 tokens = 256*K routes, owned by one 1024-thread workgroup;
-//     tiles are handed out by an atomic ticket so that every tile's predecessors
-//     have already started, which makes the look-back below deadlock-free
-//     whatever the residency of the grid; the same fetch-add returns the
-//     launch's generation, and the last ticket holder resets the word;
+//     one fetch-add per tile on the workspace's turn word returns the launch's
+//     generation and an arrival number, and the last arrival resets the word.
+//     Large grids take the arrival number as their tile, so that every tile's
+//     predecessors have already started and the look-back below cannot wait on a
+//     workgroup that is not resident; small grids (a tile per eight compute
+//     units at most) take workgroup b = tile b and need the fetch-add's answer
+//     only when they publish;
 //   * the workgroup is 16 waves; each walks its share of the tile's 4*K chunks
 //     of 64 routes in (token, slot) order;
 //     lanes holding the same expert find each other with log2(E) ballots, the
@@ -25,8 +28,8 @@
 //     single-pass decoupled look-back on 64-bit status words
 //     {flag:2 | generation:30 | value:32}; the generation tag makes the words of
 //     earlier launches invalid without any clearing pass;
-//   * the tile holding the last ticket knows every column total and emits counts
-//     and the aligned offsets.
+//   * the last tile knows every column total and emits counts and the aligned
+//     offsets.
 //
 // ep_layout_counts_kernel: the workspace-free variant behind the reference's
 // DeepepDispatchLayout::compute signature (counts and flags only).
