@@ -433,7 +433,7 @@ def main():
     # The same steps with the source rows cycling through three buffers, so that they come from
     # HBM instead of the 256 MB memory-side cache that keeps a single re-read source resident.
     # Then also with the combined output cycling through three buffers: the combine writes outputs
-    # of up to 120 MiB through into the memory-side cache, and an output buffer that is rewritten every
+    # of up to 120 MiB (and part of larger ones) through into the memory-side cache, and an output buffer that is rewritten every
     # step would never have to leave it; three of them do.
     # That case is measured under both output policies of the combine: written through (the default)
     # and streamed straight to HBM (MI_EP_COMBINE_STREAM_OUTPUT).

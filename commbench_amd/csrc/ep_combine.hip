@@ -32,9 +32,10 @@ constexpr int kCombineWaves = kCombineThreads / kWave;
 constexpr int kStagedThreads = 1024;
 constexpr int kStagedWaves = kStagedThreads / kWave;
 constexpr int kStageBytes = 160 * 1024;  // all of the CU's LDS: one workgroup per CU
-// Outputs that leave room in the memory-side cache (256 MB on this part; not reported by the
-// runtime) for an input of their own size are written through into it: a little under half of it.
-constexpr long long kStoreThroughBytesMax = 120ll * 1024 * 1024;
+// What one step may keep in the memory-side cache (256 MB on this part; not reported by the
+// runtime): the output written through into it plus an input of the output's size, which the next
+// step re-reads, have to fit.
+constexpr long long kMemorySideCacheBudget = 240ll * 1024 * 1024;
 
 // Computes one unit; out[u] holds the packed bf16 of vector v0 + u * 64 (valid
 // where that index is inside the row).
@@ -157,13 +158,14 @@ __global__ __launch_bounds__(kCombineThreads) void ep_combine_kernel(const Combi
 // in the middle of its reads (8192 x 14 KiB rows: 174 -> 164 us, whole step 346 -> 338 us).  That
 // holds while the output and an input of its size that the next step re-reads both fit that cache;
 // beyond, the dirty lines fall out during the next kernel's writes and cost it more than was gained
-// (176 MB of output: this kernel -12 us, the following copy +32 us), so larger outputs are streamed
-// ("nt") as before.
+// (176 MB of output all written through: this kernel -12 us, the following copy +32 us), so only
+// groups of tokens below `through_tokens` are written through and the rest is streamed ("nt"): with the
+// share that still fits, 16384 x 8 KiB rows gain 10 us of 388 and 12288 x 14 KiB rows 9 us of 520.
 template <int kTopk, int kRegUnits>
 __global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const CombineArgs a,
                                                                           const int group_tokens,
                                                                           const int lds_units,
-                                                                          const int store_through) {
+                                                                          const int through_tokens) {
   extern __shared__ vec16 stage[];  // [lds_units][64]
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
@@ -212,7 +214,7 @@ __global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const
         __builtin_amdgcn_make_buffer_rsrc(dst, 0, gn * a.row_vecs * static_cast<int>(sizeof(vec16)), kRawBufferFormat);
     auto store = [&](const vec16 value, const int vec_index) {
       const int offset = vec_index * static_cast<int>(sizeof(vec16));
-      if (store_through)
+      if (g0 < through_tokens)
         __builtin_amdgcn_raw_buffer_store_b128(value, group_rows, offset, 0, kCachePolicyDeviceScope);
       else
         __builtin_amdgcn_raw_buffer_store_b128(value, group_rows, offset, 0, kCachePolicyStreaming);
@@ -290,14 +292,24 @@ hipError_t launch_combine_k(const CombineArgs& a, hipStream_t stream) {
       if (e != hipSuccess) return e;
       raised.store(1, std::memory_order_release);
     }
-    const int store_through =
-        (!a.stream_output && static_cast<long long>(a.num_tokens) * row_bytes <= kStoreThroughBytesMax) ? 1 : 0;
+    // Rows written through: all of them while twice the output fits the budget, else the first
+    // whole phases that leave room for an input of the output's size (a phase in which some
+    // workgroups write through and others stream costs more than it saves: 16384 x 14 KiB rows with
+    // 16 MiB written through, +11 us), none from an output of the budget's size on.
+    const long long out_bytes = static_cast<long long>(a.num_tokens) * row_bytes;
+    long long through_bytes = kMemorySideCacheBudget - out_bytes;
+    if (through_bytes > out_bytes) through_bytes = out_bytes;
+    if (through_bytes < 0 || a.stream_output) through_bytes = 0;
+    const long long phase_tokens = static_cast<long long>(grid) * group_tokens;
+    const int through_tokens = through_bytes == out_bytes
+                                   ? a.num_tokens
+                                   : static_cast<int>(through_bytes / row_bytes / phase_tokens * phase_tokens);
     if (with_registers)
       hipLaunchKernelGGL((ep_combine_staged_kernel<kTopk, kStagedRegUnits>), dim3(grid), dim3(kStagedThreads), lds,
-                         stream, a, group_tokens, lds_units, store_through);
+                         stream, a, group_tokens, lds_units, through_tokens);
     else
       hipLaunchKernelGGL((ep_combine_staged_kernel<kTopk, 0>), dim3(grid), dim3(kStagedThreads), lds, stream, a,
-                         group_tokens, lds_units, store_through);
+                         group_tokens, lds_units, through_tokens);
     return hipGetLastError();
   }
   // Everything else: one unit per wave; two vectors per lane once rows are long.

@@ -346,10 +346,12 @@ int mi_ep_pull_indices(const int* recv_src_map, int num_rows, int tokens_per_sou
  *                written through into the GPU's memory-side cache (256 MB), where the operator
  *                that consumes it next finds it and from where it reaches HBM later; the kernel
  *                itself is then almost a pure read stream (about 5 % faster on large shapes).
- *                With the flag, and always beyond 120 MiB, the output is streamed straight to
- *                HBM: the choice for an output that nothing reads soon, since lines that fall
- *                out of that cache during other memory-bound kernels cost those more than the
- *                flag costs this one.  The results are identical.
+ *                Of a larger output only the leading part that leaves that cache room for an
+ *                input of the output's size is written through (nothing from 240 MiB on).
+ *                With the flag the whole output is streamed straight to HBM: the choice for an
+ *                output that nothing reads soon, since lines that fall out of that cache during
+ *                other memory-bound kernels cost those more than the flag costs this one.  The
+ *                results are identical.
  */
 #define MI_EP_COMBINE_STREAM_OUTPUT 1
 int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float* topk_weights,
