@@ -156,6 +156,10 @@ int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, in
   // tiles by arrival and need no such argument.  The wait is bounded either way.
   DeviceTraits dev{};
   a.static_tiles = (device_traits(s, &dev) == hipSuccess && a.num_tiles * 8 <= dev.compute_units) ? 1 : 0;
+  // Grids whose last tile can fetch every predecessor's packed row in two rounds of 16-byte loads do
+  // that instead of walking back column by column.
+  const long long row_words = (num_experts + 1) / 2 + (num_ranks + 1) / 2;
+  a.gather_rows = ((a.num_tiles - 1) * row_words <= kGatherLimitWords && aligned16(workspace)) ? 1 : 0;
   a.expert_bits = 1;
   while ((1 << a.expert_bits) < num_experts) ++a.expert_bits;
   a.inv_topk = ((1u << 19) + num_topk - 1) / num_topk;

@@ -38,6 +38,12 @@ struct alignas(256) LayoutWorkspace {
 };
 // Polls are spaced by s_sleep, roughly a microsecond apart: a few seconds before a launch gives up.
 constexpr uint32_t kDefaultWaitLimit = 1u << 22;
+// Small grids gather their predecessors' status rows whole: 16-byte loads, two in flight per lane
+// (four cost 0.7 us more at 32 tiles), so that a workgroup takes in kGatherWords status words per
+// round trip.  The rule is that the last tile's predecessors take at most two rounds.
+constexpr int kGatherDepth = 2;
+constexpr int kGatherWords = 2 * kGatherDepth * kLayoutThreads;
+constexpr int kGatherLimitWords = 2 * kGatherWords;
 
 struct LayoutArgs {
   const int64_t* topk_idx;
@@ -64,6 +70,7 @@ struct LayoutArgs {
   int num_channels;
   int num_tiles;
   int static_tiles;  // 1: workgroup b takes tile b (every workgroup is resident at once); 0: tiles by ticket
+  int gather_rows;   // 1: two columns per status word, every predecessor's row fetched at once (small grids)
   int rank_slot_base;
   int expert_bits;  // ceil(log2(num_experts)), at least 1
   uint32_t inv_topk;              // ceil(2^19 / num_topk): n / num_topk == (n * inv) >> 19 for n < 2048

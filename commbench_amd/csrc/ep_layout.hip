@@ -24,10 +24,15 @@
 //     lowest such lane bumps the wave's private LDS counter once, and every lane
 //     derives its rank among equals with a popcount -- no LDS atomics, so routing
 //     skew costs nothing;
-//   * columns (E experts followed by R ranks) are scanned across tiles with a
-//     single-pass decoupled look-back on 64-bit status words
-//     {flag:2 | generation:30 | value:32}; the generation tag makes the words of
-//     earlier launches invalid without any clearing pass;
+//   * columns (E experts followed by R ranks) are scanned across tiles in a single
+//     pass over 64-bit status words {flag:2 | generation:30 | value:32}; the
+//     generation tag makes the words of earlier launches invalid without any
+//     clearing pass.  Small grids (the last tile's predecessors amount to at most
+//     kGatherLimitWords words) publish two 16-bit column totals per word and every
+//     tile fetches all its predecessors' rows at once, as one contiguous run read
+//     with 16-byte loads by the whole workgroup and summed with LDS adds; larger
+//     grids publish one column per word and walk back column by column (decoupled
+//     look-back: aggregates until a tile's inclusive prefix is met);
 //   * the last tile knows every column total and emits counts and the aligned
 //     offsets.
 //
@@ -48,6 +53,9 @@ constexpr int kCountsThreads = 1024;  // the counts-only kernel: one token per t
 __device__ __forceinline__ uint64_t pack_status(uint32_t flag, uint32_t gen, uint32_t value) {
   return (static_cast<uint64_t>(flag) << 62) | (static_cast<uint64_t>(gen & kGenMask) << 32) |
          static_cast<uint64_t>(value);
+}
+__device__ __forceinline__ uint32_t pack_pair(int first, int second) {
+  return (static_cast<uint32_t>(first) & 0xffffu) | (static_cast<uint32_t>(second) << 16);
 }
 __device__ __forceinline__ void publish(uint64_t* p, uint64_t v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -99,6 +107,9 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
   uint64_t* status = reinterpret_cast<uint64_t*>(a.ws + 1);
+  // Small grids pack two columns into a status word: experts first, then ranks.
+  const int expert_words = (E + 1) >> 1;
+  const int row_words = expert_words + ((R + 1) >> 1);
 
   // ---- routes: the tile's 256*K routes are 4*K chunks of 64 in (token, slot)
   // order; wave w owns chunks [w * per_wave, (w + 1) * per_wave).
@@ -153,6 +164,8 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     for (int i = tid; i < (kLayoutWaves * E + 1) / 2; i += kLayoutThreads) hist_words[i] = 0;
   }
   if (tid < kTileTokens) tok_flags[tid] = 0;
+  if (a.gather_rows)  // the gathered look-back adds into these
+    for (int i = tid; i < cols; i += kLayoutThreads) col_excl[i] = 0;
   __syncthreads();
 
   const int tile = a.static_tiles ? static_cast<int>(blockIdx.x) : misc[0];
@@ -222,8 +235,17 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     }
     col_total[col] = total;
     my_col_total = total;
-    publish(status + static_cast<size_t>(tile) * cols + col,
-            pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
+    if (a.gather_rows) {
+      // Two columns per word (a tile holds at most 256 * 8 routes, so 16 bits each): the even
+      // lane takes its neighbour's total and publishes for both.
+      const int neighbour = __builtin_amdgcn_update_dpp(0, total, 0x101, 0xf, 0xf, false);  // row_shl:1
+      if ((col & 1) == 0)
+        publish(status + static_cast<size_t>(tile) * row_words + (col >> 1),
+                pack_status(kFlagAggregate, gen, pack_pair(total, col + 1 < E ? neighbour : 0)));
+    } else {
+      publish(status + static_cast<size_t>(tile) * cols + col,
+              pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
+    }
   }
   // Exclusive scan of the tile's per-expert counts (one expert per thread): where each expert's
   // routes start in the tile's route order.  The cross-wave half follows the next barrier.
@@ -266,8 +288,15 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
 #pragma unroll
     for (int w = 0; w < kTileTokens / kWave; ++w) total += rank_wave[w * kMaxRanks + tid];
     col_total[E + tid] = total;
-    publish(status + static_cast<size_t>(tile) * cols + E + tid,
-            pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
+    if (a.gather_rows) {
+      const int neighbour = __builtin_amdgcn_update_dpp(0, total, 0x101, 0xf, 0xf, false);  // row_shl:1
+      if ((tid & 1) == 0)
+        publish(status + static_cast<size_t>(tile) * row_words + expert_words + (tid >> 1),
+                pack_status(kFlagAggregate, gen, pack_pair(total, tid + 1 < R ? neighbour : 0)));
+    } else {
+      publish(status + static_cast<size_t>(tile) * cols + E + tid,
+              pack_status(tile == 0 ? kFlagPrefix : kFlagAggregate, gen, static_cast<uint32_t>(total)));
+    }
     if (a.tile_rank_counts != nullptr) a.tile_rank_counts[static_cast<size_t>(tile) * R + tid] = total;
   }
   // In the shadow of the publication: the flags go out and the cross-wave half of the route-order
@@ -319,8 +348,57 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     }
   }
 
-  // ---- the decoupled look-back of every column ----------------------------------
-  for (int col = tid; col < cols; col += kLayoutThreads) {
+  // ---- small grids: every predecessor's row gathered at once ---------------------
+  // The rows of tiles 0 .. tile-1 are one contiguous run of tile * row_words status words.  The
+  // whole workgroup fetches it, two words (four columns) per lane and load, and adds what it finds
+  // to the columns' sums in LDS: a tile with 31 predecessors issues two loads per wave where a
+  // column-per-thread walk issues 31, and a device-scope load costs by the instruction, not by
+  // the byte.
+  if (a.gather_rows) {
+    const int words = tile * row_words;
+    const __amdgpu_buffer_rsrc_t rows = __builtin_amdgcn_make_buffer_rsrc(status, 0, (words + 1) * 8, kRawBufferFormat);
+    auto fold = [&](const uint32_t lo, const uint32_t hi, const int word) -> bool {
+      if ((hi & kGenMask) != gen || (hi >> 30) == 0) return false;
+      const int w = word % row_words;
+      const int col = w < expert_words ? 2 * w : E + 2 * (w - expert_words);
+      // A column that does not exist (odd E or R) was published as zero.
+      if ((lo & 0xffffu) != 0) atomicAdd(&col_excl[col], static_cast<int>(lo & 0xffffu));
+      if ((lo >> 16) != 0) atomicAdd(&col_excl[col + 1], static_cast<int>(lo >> 16));
+      return true;
+    };
+    for (int first = 0; first < words; first += kGatherWords) {
+      vec16 got[kGatherDepth];
+#pragma unroll
+      for (int d = 0; d < kGatherDepth; ++d) {
+        const int word = first + 2 * (d * kLayoutThreads + tid);
+        got[d] = vec16{0u, 0u, 0u, 0u};
+        if (word < words) got[d] = __builtin_amdgcn_raw_buffer_load_b128(rows, word * 8, 0, kCachePolicyDeviceScope);
+      }
+#pragma unroll
+      for (int d = 0; d < kGatherDepth; ++d) {
+        const int word = first + 2 * (d * kLayoutThreads + tid);
+        bool need_0 = word < words, need_1 = word + 1 < words;
+        uint32_t spins = 0;
+        vec16 v = got[d];
+        while (true) {
+          if (need_0 && fold(v.x, v.y, word)) need_0 = false;
+          if (need_1 && fold(v.z, v.w, word + 1)) need_1 = false;
+          if (!need_0 && !need_1) break;
+          if (++spins >= wait_limit) {
+            __hip_atomic_store(&a.ws->timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (a.timeout_report != nullptr)
+              __hip_atomic_store(a.timeout_report, kTimedOutCode, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
+          v = __builtin_amdgcn_raw_buffer_load_b128(rows, word * 8, 0, kCachePolicyDeviceScope);
+        }
+      }
+    }
+  }
+
+  // ---- larger grids: the decoupled look-back of every column ----------------------
+  for (int col = tid; col < cols && !a.gather_rows; col += kLayoutThreads) {
     const int total = col_total[col];
     uint64_t* mine = status + static_cast<size_t>(tile) * cols + col;
     int excl = 0;

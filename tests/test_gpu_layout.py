@@ -84,6 +84,27 @@ def test_fused_layout_ragged_shapes(oracle, shape):
     gu.check_layout_against_oracle(oracle, h, topk_np, R, E, 3, 5)
 
 
+@pytest.mark.parametrize("shape", [
+    (4096, 4, 8, 1024), (4097, 4, 8, 1024), (2304, 2, 8, 1024), (2000, 8, 3, 3), (8192, 8, 1, 1), (16384, 3, 7, 7)],
+    ids=lambda s: "x".join(map(str, s)))
+def test_fused_layout_gathered_and_walked_scans(oracle, shape):
+    """Small grids fetch every predecessor's packed status row at once, larger ones walk back column
+    by column: 1024 experts x 8 ranks change over between 16 and 17 tiles (4096 / 4097 tokens) and
+    need one round of loads up to 8 predecessors (2304 tokens) and two beyond; odd expert and rank
+    counts leave half a status word empty; a token whose slots all name one expert drives a column
+    to the 2048 routes per tile that its 16 bits must hold."""
+    T, K, R, E = shape
+    print(f"shape {shape}", flush=True)
+    rng = np.random.default_rng(T + E)
+    topk_np = rng.integers(-1, E, size=(T, K)).astype(np.int64)
+    if E <= 3:
+        topk_np[: T // 2] = E - 1                        # whole tiles on one expert
+    buf = ops.Buffer(T, K, E, R, device=gu.DEV)
+    for _ in range(2):
+        _, h = gu.run_fused_layout(buf, topk_np, expert_alignment=2, num_channels=3)
+    gu.check_layout_against_oracle(oracle, h, topk_np, R, E, 2, 3)
+
+
 @pytest.mark.parametrize("shape", [(300000, 2, 8, 64), (131072, 8, 8, 256)], ids=lambda s: "x".join(map(str, s)))
 def test_fused_layout_more_tiles_than_resident_workgroups(oracle, shape):
     """Over a thousand tiles: more workgroups than the device holds at once.  Tiles are handed out
