@@ -153,6 +153,18 @@ def test_workspace_is_reusable_across_shapes_and_many_calls(oracle):
         gu.check_layout_against_oracle(oracle, h, topk_np, R, E)
 
 
+def test_workspace_alternates_between_gathered_and_walked_scans(oracle):
+    """One workspace, 1024 experts: launches of up to 16 tiles pack two columns per status word, larger
+    ones keep one; words left by the other form must never be taken for this launch's."""
+    K, R, E = 4, 8, 1024
+    buf = ops.Buffer(8192, K, E, R, device=gu.DEV)
+    rng = np.random.default_rng(23)
+    for T in [4096, 8192, 2304, 8192, 4096, 300, 8192, 4096]:
+        topk_np = rng.integers(-1, E, size=(T, K)).astype(np.int64)
+        _, h = gu.run_fused_layout(buf, topk_np, expert_alignment=4, num_channels=8)
+        gu.check_layout_against_oracle(oracle, h, topk_np, R, E, 4, 8)
+
+
 @pytest.mark.parametrize("T", [7, 4096, 4097])
 @pytest.mark.parametrize("R", [2, 4, 8])
 def test_channel_prefix_reference_notify_cases(oracle, T, R):
@@ -167,13 +179,16 @@ def test_channel_prefix_reference_notify_cases(oracle, T, R):
     np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy(), oracle.channel_prefix(flags, C))
 
 
-def test_expired_wait_terminates_and_is_reported(oracle):
+@pytest.mark.parametrize("shape", [(65536, 8, 8, 256), (262144, 2, 8, 8)], ids=["walked", "gathered"])
+def test_expired_wait_terminates_and_is_reported(oracle, shape):
     """Failure handling without a hang: with the wait limit forced to one poll, a launch over many
-    tiles gives up at least one look-back wait; it must still finish, the workspace must report
-    it, and after re-initialisation the same workspace must work again."""
+    tiles gives up at least one wait of its scan (256 tiles walking back column by column; 1024 tiles
+    of 16 columns gathering their predecessors' rows); it must still finish, the workspace must
+    report it, and after re-initialisation the same workspace must work again."""
     from commbench_amd import _lib
     lib = _lib.load()
-    T, K, R, E = 65536, 8, 8, 256
+    T, K, R, E = shape
+    print(f"shape {shape}", flush=True)
     topk_np = wl.uniform_distinct_topk(np.random.default_rng(3), T, E, K)
     topk = torch.from_numpy(topk_np).to(gu.DEV)
     buf = ops.Buffer(T, K, E, R, device=gu.DEV)
@@ -188,7 +203,7 @@ def test_expired_wait_terminates_and_is_reported(oracle):
                 assert code == -110 and _lib.strerror(code) == "device-side wait timed out"
                 expired = True
                 break
-        assert expired, "no wait expired with a one-poll limit over 256 tiles"
+        assert expired, "no wait expired with a one-poll limit over hundreds of tiles"
         with pytest.raises(_lib.MiEpError):
             buf.status()
     finally:
