@@ -60,6 +60,9 @@ int mi_ep_get_dispatch_layout(const int64_t* topk_idx, int* num_tokens_per_rank,
  * Workspace of the fused layout kernel below.  It must be initialised once
  * (mi_ep_workspace_init) before its first use; every later call leaves it ready
  * for the next.  Calls that share one workspace must not overlap in time.
+ * It must be 8-byte aligned; with 16-byte alignment (any hipMalloc result) grids
+ * of up to a few dozen tiles scan their tiles' totals with wide loads, which is
+ * about 2 us faster per launch.
  */
 size_t mi_ep_workspace_bytes(int num_tokens, int num_topk, int num_experts, int num_ranks);
 int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
