@@ -148,7 +148,7 @@ int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, in
   a.num_channels = num_channels;
   a.num_tiles = num_tiles_for(num_tokens);
   // Small grids take static tiles (workgroup b = tile b: one memory round trip less before the first
-  // load).  A look-back then may wait on a tile whose workgroup has not started, which is harmless as
+  // load).  A tile's scan then may wait on a tile whose workgroup has not started, which is harmless as
   // long as that workgroup finds a slot: with at most one tile per eight compute units a launch takes
   // 1/16 of the slots its workgroups could occupy (two fit a compute unit), so that sixteen such
   // launches would have to execute at once, each partly resident, before one could keep another's
