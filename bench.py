@@ -654,8 +654,14 @@ def main():
             us = time_steps(torch, owk, 60, 100) * 1e6      # 60 steps: past the clock ramp that follows idle
             omarks = kernel_medians(torch, owk, 30)
             median = lambda i: sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for ev in omarks)[len(omarks) // 2]
+            # cost of one event record, as for the headline: bracketed steps against plain steps
+            bracketed_us = omarks[0][0].elapsed_time(omarks[-1][3]) * 1e3
+            record_us = min(5.0, max(0.0, (bracketed_us - us * len(omarks)) / (4 * len(omarks) - 1)))
             entry = {"us_per_step": us, "tokens_per_s": ocfg.num_tokens / (us * 1e-6),
                      "kernel_us_median": {"layout": median(0), "dispatch": median(1), "combine": median(2)},
+                     "event_record_us": record_us,
+                     "kernel_us_median_net": {"layout": median(0) - record_us, "dispatch": median(1) - record_us,
+                                              "combine": median(2) - record_us},
                      "algorithmic_bytes": owk.bytes["total"],
                      "hbm_gbps_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9,
                      "hbm_frac_whole_step": owk.bytes["total"] / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS}
