@@ -28,8 +28,8 @@ STREAM_OUTPUT = 1           # MI_EP_COMBINE_STREAM_OUTPUT
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="target")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
@@ -48,6 +48,10 @@ def parse_args():
     ap.add_argument("--no-yardsticks", action="store_true",
                     help="skip the linear copy / read / write streams measured beside the roofline")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--sustained-steps", type=int, default=3000,
+                    help="back-to-back steps of each sustained-load leg, timed in windows of "
+                         "--sustained-window steps (0 skips the legs)")
+    ap.add_argument("--sustained-window", type=int, default=100)
     ap.add_argument("--schedule-sweep", action="store_true",
                     help="instead of the benchmark: time the dispatch copy under both schedules over a grid of row "
                          "sizes and token counts (the table the automatic choice is derived from) and print it as JSON")
@@ -111,6 +115,7 @@ class Workload:
         self.in_rank = torch.empty((T, R), dtype=torch.bool, device=dev)
         self.off = torch.empty(E + 1, **i32)
         self.psum = torch.empty(R, **i32)
+        self.rank_prefix = torch.empty((R, R), **i32)
         self.slot_rel = torch.empty((T, K), **i32)
         self.slot_map = torch.empty((T, K), **i32)
         self.route_order = torch.empty((self.lib.mi_ep_route_order_bytes(T, K) // 16, 4), **i32)
@@ -139,8 +144,9 @@ class Workload:
         self._lib.check(self.lib.mi_ep_dispatch_layout(
             self.topk.data_ptr(), c.num_tokens, c.num_topk, c.num_ranks, c.num_experts, self.align, 0,
             self.per_rank.data_ptr(), self.per_expert.data_ptr(), self.in_rank.data_ptr(),
-            self.off.data_ptr(), self.psum.data_ptr(), None, self.slot_rel.data_ptr(), None, 0,
-            self.route_order.data_ptr(), None, None, None, self.ws.data_ptr(), self.ws.numel(), self.stream),
+            self.off.data_ptr(), self.psum.data_ptr(), None, self.rank_prefix.data_ptr(), self.slot_rel.data_ptr(),
+            None, 0, self.route_order.data_ptr(), None, None, None, self.ws.data_ptr(), self.ws.numel(),
+            self.stream),
             "layout")
 
     def dispatch(self):
@@ -218,7 +224,7 @@ class RankWorkload:
         self._lib.check(self.lib.mi_ep_dispatch_layout(
             self.topk.data_ptr(), c.num_tokens, c.num_topk, c.num_ranks, c.num_experts, 1, 0,
             self.per_rank.data_ptr(), self.per_expert.data_ptr(), self.in_rank.data_ptr(), None, None, None, None,
-            self.rank_slot_idx.data_ptr(), 0, None, None, None, None, self.ws.data_ptr(), self.ws.numel(),
+            None, self.rank_slot_idx.data_ptr(), 0, None, None, None, None, self.ws.data_ptr(), self.ws.numel(),
             self.stream), "layout")
 
     def dispatch(self):
@@ -326,19 +332,24 @@ def source_fingerprint(path):
     return hashlib.sha256(" ".join(text.split()).encode()).hexdigest()[:16]
 
 
-def measured_traffic(kernel, workload_name):
-    """HBM bytes per launch of `kernel` from the committed counter runs, or None when the kernel
-    sources have changed since they were taken (the file records their fingerprints)."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+TRAFFIC_FILE = "profiles/hbm_traffic.json"
+
+
+def profiled_record(workload_name):
+    """What the committed counter and trace runs hold for a workload: {"traffic": {kernel: HBM bytes
+    per launch}, "profiled_us": {kernel: average duration of the timed region's dispatches under
+    rocprofv3}}; empty when the kernel sources have changed since they were taken (the file records
+    their fingerprints).  Read from a committed file, not measured in this run."""
+    path = os.path.join(ROOT, TRAFFIC_FILE)
     if not os.path.exists(path):
-        return None
+        return {}
     with open(path) as f:
         rec = json.load(f)
     for name, want in rec.get("source_sha16", {}).items():
         src = os.path.join(ROOT, "commbench_amd", "csrc", name)
         if not os.path.exists(src) or source_fingerprint(src) != want:
-            return None
-    return rec.get(workload_name, {}).get(kernel)
+            return {}
+    return {"traffic": rec.get(workload_name, {}), "profiled_us": rec.get("profiled_us", {}).get(workload_name, {})}
 
 
 def time_steps(torch, wk, warmup, steps):
@@ -350,6 +361,31 @@ def time_steps(torch, wk, warmup, steps):
         wk.step()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) / steps
+
+
+def sustained_leg(torch, wk, total_steps, window):
+    """`total_steps` steps back to back on the launch stream with one HIP event every `window`
+    steps: the fraction of peak HBM bandwidth (algorithmic bytes of the whole step) of every
+    window, so that a throughput that only holds for milliseconds shows."""
+    windows = max(1, total_steps // window)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(windows + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    marks[0].record()
+    for i in range(windows):
+        for _ in range(window):
+            wk.step()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    us = [marks[i].elapsed_time(marks[i + 1]) * 1e3 / window for i in range(windows)]
+    frac = [wk.bytes["total"] / (u * 1e-6) / 1e9 / PEAK_HBM_GBPS for u in us]
+    ordered = sorted(frac)
+    return {"steps": windows * window, "window_steps": window, "seconds": seconds,
+            "us_per_step_median": sorted(us)[len(us) // 2], "us_per_step_max": max(us),
+            "hbm_frac_first_window": frac[0], "hbm_frac_median_window": ordered[len(ordered) // 2],
+            "hbm_frac_min_window": ordered[0], "hbm_frac_last_window": frac[-1],
+            "min_window_index": frac.index(ordered[0])}
 
 
 def kernel_medians(torch, wk, reps):
@@ -438,6 +474,7 @@ def main():
     # That case is measured under both output policies of the combine: written through (the default)
     # and streamed straight to HBM (MI_EP_COMBINE_STREAM_OUTPUT).
     cold_ms_per_step = cold_both_ms_per_step = cold_both_streamed_ms_per_step = None
+    cold_both_marks = sustained_hot = sustained_cold = sustained_cold_streamed = None
     if len(wk.x_ring) == 1 and not args.no_cold_source:
         ring = wk.x_ring
         wk.x_ring = [wk.x, wk.x.clone(), wk.x.clone()]
@@ -455,13 +492,20 @@ def main():
         cold_ms_per_step = cold_pass()
         wk.out_ring = [wk.out, torch.empty_like(wk.out), torch.empty_like(wk.out)]
         cold_both_ms_per_step = cold_pass()
+        cold_both_marks = kernel_medians(torch, wk, args.steps)
+        if args.sustained_steps > 0:
+            sustained_cold = sustained_leg(torch, wk, args.sustained_steps, args.sustained_window)
         wk.combine_flags = STREAM_OUTPUT
         cold_both_streamed_ms_per_step = cold_pass()
+        if args.sustained_steps > 0:
+            sustained_cold_streamed = sustained_leg(torch, wk, args.sustained_steps, args.sustained_window)
         wk.combine_flags = 0
         wk.x_ring = ring
         wk.out_ring = [wk.out]
         wk.step()
         torch.cuda.synchronize()
+    if args.sustained_steps > 0:
+        sustained_hot = sustained_leg(torch, wk, args.sustained_steps, args.sustained_window)
 
     # The same steps replayed as one HIP graph of the three kernels (no host launch gaps).
     graph_ms_per_step = None
@@ -561,8 +605,32 @@ def main():
     records = 4 * len(marks) - 1
     event_record_us = min(5.0, max(0.0, (bracketed_step_us - ms_per_step * 1e3) * len(marks) / records))
     kernel_us_net = {n: kernel_us[n] - event_record_us for n in names}
-    dominant = max(names, key=lambda n: kernel_us[n])
-    achieved = kernel_bytes[dominant] / (kernel_us_net[dominant] * 1e-6) / 1e9
+    # The roofline is taken on the RAW intervals (kernel + launch gap + one event record): they can
+    # only overstate a kernel's duration, so the fraction is a lower bound that the profiler's own
+    # durations (profiled_us, from the committed trace) must not fall below.  Both hot kernels are
+    # reported; the line's headline kernel is the slower of the two in this run.
+    profiled = profiled_record(cfg.name)
+    hot = names[1:]
+    dominant = max(hot, key=lambda n: kernel_us[n])
+    gbps = lambda n, us: kernel_bytes[n] / (us * 1e-6) / 1e9
+
+    def kernel_entry(n):
+        entry = {"algorithmic_bytes": kernel_bytes[n], "us_raw": kernel_us[n], "us_net": kernel_us_net[n],
+                 "frac_raw": gbps(n, kernel_us[n]) / PEAK_HBM_GBPS, "frac_net": gbps(n, kernel_us_net[n]) / PEAK_HBM_GBPS,
+                 "traffic": profiled.get("traffic", {}).get(n), "profiled_us": profiled.get("profiled_us", {}).get(n)}
+        if entry["profiled_us"]:
+            entry["frac_profiled"] = gbps(n, entry["profiled_us"]) / PEAK_HBM_GBPS
+        return entry
+
+    roofline_kernels = {n: kernel_entry(n) for n in hot}
+    achieved = gbps(dominant, kernel_us[dominant])
+    # The same intervals with the source rows and the output cycling through three buffers each:
+    # nothing counted stays in the memory-side cache from one step to the next.
+    all_hbm = None
+    if cold_both_marks is not None:
+        cold_us = {n: sum(ev[i + 1].elapsed_time(ev[i + 2]) * 1e3 for ev in cold_both_marks) / len(cold_both_marks)
+                   for i, n in enumerate(hot)}
+        all_hbm = {n: {"us_raw": cold_us[n], "frac_raw": gbps(n, cold_us[n]) / PEAK_HBM_GBPS} for n in hot}
 
     result = {
         "metric": "dispatch+combine tokens/s and achieved HBM GB/s (% of peak), 1 MI355X",
@@ -618,11 +686,31 @@ def main():
         "write_yardstick_gbps": write_gbps,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBPS,
-                     "duration_us": kernel_us_net[dominant],
-                     "timing": "average HIP-event interval around the kernel over the steps, less the measured "
-                               "cost of one event record (event_record_us); the launch gap stays in",
-                     "traffic": measured_traffic(dominant, cfg.name)},
+                     "duration_us": kernel_us[dominant],
+                     "timing": "average raw HIP-event interval around the kernel over the timed steps: the kernel, "
+                               "its launch gap and one event record (frac_net in `kernels` subtracts the measured "
+                               "cost of a record, event_record_us; profiled_us / frac_profiled are the dispatches' "
+                               "own durations under rocprofv3, from the committed trace)",
+                     "traffic": roofline_kernels[dominant]["traffic"],
+                     "traffic_source": TRAFFIC_FILE + " (two rocprofv3 --pmc runs, committed; not measured in this "
+                                                      "run; null when the kernel sources have changed since)",
+                     "kernels": roofline_kernels,
+                     "cache_assisted": "in the timed region the single source buffer (re-read every step) and the "
+                                       "combine's output (rewritten every step, written through) stay in the "
+                                       "256 MB memory-side cache; all_bytes_cross_hbm repeats the intervals with "
+                                       "both cycling through three buffers",
+                     "all_bytes_cross_hbm": all_hbm},
     }
+    if sustained_hot is not None:
+        sustained = dict(sustained_hot)
+        if sustained_cold is not None:
+            sustained["cold_both"] = dict(sustained_cold, output_policy="written through (default)")
+            sustained["cold_both_streamed"] = dict(sustained_cold_streamed,
+                                                   output_policy="streamed (MI_EP_COMBINE_STREAM_OUTPUT)")
+        sustained["note"] = ("steps back to back on one stream, one HIP event per window; fractions are "
+                             "algorithmic bytes of the whole step against 8 TB/s; cold_both: source rows and "
+                             "combined output each cycling through three buffers")
+        result["sustained"] = sustained
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, wk, args.cpu_seconds)
     if not args.no_host_path:

@@ -22,10 +22,10 @@ SIGNATURES = {
     "mi_ep_device_traits": (_int, [_c_int_p, _c_int_p, _c_int_p, _vp]),
     "mi_ep_dispatch_schedule_for": (_int, [_int, _int, _int, _int, _int, _int]),
     "mi_ep_dispatch_layout": (_int, [_vp, _int, _int, _int, _int, _int, _int,
-                                     _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp,
+                                     _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp,
                                      _vp, _size, _vp]),
     "mi_ep_dispatch_layout_static": (_int, [_vp, _int, _int, _int, _int, _int, _int,
-                                            _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp,
+                                            _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp,
                                             _vp, _vp]),
     "mi_ep_route_order_bytes": (_size, [_int, _int]),
     "mi_ep_dispatch": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int,
@@ -46,7 +46,7 @@ SIGNATURES = {
     "mi_ep_combine": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp, _int, _vp]),
     "mi_ep_host_get_dispatch_layout": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int]),
     "mi_ep_host_dispatch_layout": (_int, [_vp, _int, _int, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp,
-                                          _vp, _vp, _int, _vp, _vp, _vp, _vp]),
+                                          _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp]),
     "mi_ep_host_dispatch": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _int,
                                    _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int]),
     "mi_ep_host_dispatch_ranks": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _int, _int,
@@ -57,6 +57,8 @@ SIGNATURES = {
     "mi_ep_read_yardstick": (_int, [_vp, _size, _vp, _vp]),
     "mi_ep_write_yardstick": (_int, [_vp, _size, _vp]),
 }
+
+STATIC_SCRATCH = 256   # MI_EP_STATIC_SCRATCH: the library's own layout scratch, for the workspace calls
 
 _lib = None
 

@@ -50,17 +50,30 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
 // Device address of `scratch` per device ordinal: resolved on the first call on that device,
-// read-only afterwards (every resolver stores the same value).
+// read-only afterwards (every resolver stores the same value).  Like any device address it does not
+// outlive a hipDeviceReset of that device.
 std::atomic<void*> g_scratch_address[kMaxDevices];
 
-int static_scratch_of_current_device(void** out) {
+// The static scratch of the device `stream` belongs to (of the current device for the null
+// stream): the device the kernels are launched on, whatever device is current.
+int static_scratch_of(hipStream_t stream, void** out) {
   int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
+  hipError_t e = stream != nullptr ? hipStreamGetDevice(stream, &dev) : hipGetDevice(&dev);
   if (e != hipSuccess) return static_cast<int>(e);
   if (dev < 0 || dev >= kMaxDevices) return MI_EP_EINVAL;
   void* p = g_scratch_address[dev].load(std::memory_order_acquire);
   if (p == nullptr) {
+    // A symbol resolves to the current device's copy of the array: make the stream's device
+    // current for the lookup, and put the caller's back.
+    int current = -1;
+    e = hipGetDevice(&current);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (current != dev && (e = hipSetDevice(dev)) != hipSuccess) return static_cast<int>(e);
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (current != dev) {
+      const hipError_t back = hipSetDevice(current);
+      if (e == hipSuccess) e = back;
+    }
     if (e != hipSuccess) return static_cast<int>(e);
     if (p == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
     g_scratch_address[dev].store(p, std::memory_order_release);
@@ -69,14 +82,23 @@ int static_scratch_of_current_device(void** out) {
   return MI_EP_OK;
 }
 
+// The workspace calls take MI_EP_STATIC_SCRATCH for the library's own scratch.
+int resolve_workspace(void** workspace, size_t* workspace_bytes, hipStream_t stream) {
+  if (*workspace != MI_EP_STATIC_SCRATCH) return MI_EP_OK;
+  const int rc = static_scratch_of(stream, workspace);
+  if (rc == MI_EP_OK && workspace_bytes != nullptr) *workspace_bytes = kStaticScratchBytes;
+  return rc;
+}
+
 // Argument checks and launch shared by mi_ep_dispatch_layout (caller's workspace) and
 // mi_ep_dispatch_layout_static (workspace == nullptr and use_static_scratch: the library's static
-// scratch of the current device, resolved after the argument checks).
+// scratch on the stream's device, resolved after the argument checks).
 int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
                        int num_experts, int expert_alignment, int num_channels,
                        int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
                        int* expert_offsets, int* psum_rank_rows, int* channel_prefix_matrix,
-                       int* slot_rel, int* rank_slot_idx, int rank_slot_base, int* route_order,
+                       int* rank_prefix_matrix, int* slot_rel, int* rank_slot_idx, int rank_slot_base,
+                       int* route_order,
                        int* tile_rank_counts, int64_t* copied_topk_idx, int* cumulative_expert_stats,
                        void* workspace, size_t workspace_bytes, bool use_static_scratch,
                        int* timeout_report, void* stream) {
@@ -97,7 +119,7 @@ int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, in
   if (!aligned16(route_order)) return MI_EP_EINVAL;
   hipStream_t s = as_stream(stream);
   if (use_static_scratch && num_tokens > 0) {
-    const int rc = static_scratch_of_current_device(&workspace);
+    const int rc = static_scratch_of(s, &workspace);
     if (rc != MI_EP_OK) return rc;
     workspace_bytes = kStaticScratchBytes;
   }
@@ -114,6 +136,9 @@ int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, in
     if (e == hipSuccess && channel_prefix_matrix != nullptr)
       e = launch_fill_u32(reinterpret_cast<uint32_t*>(channel_prefix_matrix),
                           static_cast<size_t>(num_ranks) * num_channels, 0u, s);
+    if (e == hipSuccess && rank_prefix_matrix != nullptr)
+      e = launch_fill_u32(reinterpret_cast<uint32_t*>(rank_prefix_matrix),
+                          static_cast<size_t>(num_ranks) * num_ranks, 0u, s);
     return status_of(e);
   }
 
@@ -130,6 +155,7 @@ int dispatch_layout_on(const int64_t* topk_idx, int num_tokens, int num_topk, in
   a.expert_offsets = expert_offsets;
   a.psum_rank_rows = psum_rank_rows;
   a.channel_prefix_matrix = channel_prefix_matrix;
+  a.rank_prefix_matrix = rank_prefix_matrix;
   a.slot_rel = slot_rel;
   a.rank_slot_idx = rank_slot_idx;
   a.rank_slot_base = rank_slot_base;
@@ -206,6 +232,8 @@ size_t mi_ep_workspace_bytes(int num_tokens, int num_topk, int num_experts, int 
 }
 
 int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = resolve_workspace(&workspace, &workspace_bytes, as_stream(stream));
+  if (rc != MI_EP_OK) return rc;
   if (workspace == nullptr || workspace_bytes < sizeof(LayoutWorkspace)) return MI_EP_EINVAL;
   if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
   return status_of(launch_fill_u32(static_cast<uint32_t*>(workspace), workspace_bytes / 4, 0u,
@@ -213,15 +241,20 @@ int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream) 
 }
 
 int mi_ep_workspace_set_wait_limit(void* workspace, unsigned int max_polls, void* stream) {
+  const int rc = resolve_workspace(&workspace, nullptr, as_stream(stream));
+  if (rc != MI_EP_OK) return rc;
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return MI_EP_EINVAL;
   LayoutWorkspace* ws = static_cast<LayoutWorkspace*>(workspace);
   return status_of(launch_fill_u32(&ws->wait_limit, 1, max_polls, as_stream(stream)));
 }
 
 int mi_ep_workspace_status(const void* workspace, void* stream) {
-  if (workspace == nullptr) return MI_EP_EINVAL;
+  void* ws = const_cast<void*>(workspace);
+  const int rc = resolve_workspace(&ws, nullptr, as_stream(stream));
+  if (rc != MI_EP_OK) return rc;
+  if (ws == nullptr) return MI_EP_EINVAL;
   LayoutWorkspace header;
-  hipError_t e = hipMemcpyAsync(&header, workspace, sizeof(uint64_t) * 2, hipMemcpyDeviceToHost,
+  hipError_t e = hipMemcpyAsync(&header, ws, sizeof(uint64_t) * 2, hipMemcpyDeviceToHost,
                                 as_stream(stream));
   if (e != hipSuccess) return static_cast<int>(e);
   e = hipStreamSynchronize(as_stream(stream));
@@ -264,13 +297,14 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
                           int num_experts, int expert_alignment, int num_channels,
                           int* num_tokens_per_rank, int* num_tokens_per_expert,
                           bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
-                          int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
-                          int rank_slot_base, int* route_order, int* tile_rank_counts,
+                          int* channel_prefix_matrix, int* rank_prefix_matrix, int* slot_rel,
+                          int* rank_slot_idx, int rank_slot_base, int* route_order, int* tile_rank_counts,
                           int64_t* copied_topk_idx, int* cumulative_expert_stats, void* workspace,
                           size_t workspace_bytes, void* stream) {
   return dispatch_layout_on(topk_idx, num_tokens, num_topk, num_ranks, num_experts, expert_alignment,
                             num_channels, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank,
-                            expert_offsets, psum_rank_rows, channel_prefix_matrix, slot_rel, rank_slot_idx,
+                            expert_offsets, psum_rank_rows, channel_prefix_matrix, rank_prefix_matrix,
+                            slot_rel, rank_slot_idx,
                             rank_slot_base, route_order, tile_rank_counts, copied_topk_idx,
                             cumulative_expert_stats, workspace, workspace_bytes, false, nullptr, stream);
 }
@@ -279,16 +313,17 @@ int mi_ep_dispatch_layout_static(const int64_t* topk_idx, int num_tokens, int nu
                                  int num_experts, int expert_alignment, int num_channels,
                                  int* num_tokens_per_rank, int* num_tokens_per_expert,
                                  bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
-                                 int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
-                                 int rank_slot_base, int* route_order, int* tile_rank_counts,
-                                 int64_t* copied_topk_idx, int* cumulative_expert_stats,
-                                 int* timeout_report, void* stream) {
+                                 int* channel_prefix_matrix, int* rank_prefix_matrix, int* slot_rel,
+                                 int* rank_slot_idx, int rank_slot_base, int* route_order,
+                                 int* tile_rank_counts, int64_t* copied_topk_idx,
+                                 int* cumulative_expert_stats, int* timeout_report, void* stream) {
   // Nothing needs clearing between calls: the scratch starts zeroed when the code object is
   // loaded (an initialised workspace), and every launch leaves the ticket word ready for the
   // next and tags its status words with a fresh generation.
   return dispatch_layout_on(topk_idx, num_tokens, num_topk, num_ranks, num_experts, expert_alignment,
                             num_channels, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank,
-                            expert_offsets, psum_rank_rows, channel_prefix_matrix, slot_rel, rank_slot_idx,
+                            expert_offsets, psum_rank_rows, channel_prefix_matrix, rank_prefix_matrix,
+                            slot_rel, rank_slot_idx,
                             rank_slot_base, route_order, tile_rank_counts, copied_topk_idx,
                             cumulative_expert_stats, nullptr, 0, true, timeout_report, stream);
 }

@@ -53,6 +53,7 @@ struct LayoutArgs {
   int* expert_offsets;
   int* psum_rank_rows;
   int* channel_prefix_matrix;
+  int* rank_prefix_matrix;  // [R][R] or null: [source chunk][rank], inclusive over source chunks
   int* slot_rel;
   int* rank_slot_idx;
   int* route_order;  // [num_tiles * kTileTokens * K][4] or null

@@ -93,8 +93,9 @@ int mi_ep_host_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_
                                int num_experts, int expert_alignment, int num_channels,
                                int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
                                int* expert_offsets, int* psum_rank_rows, int* channel_prefix_matrix,
-                               int* slot_rel, int* rank_slot_idx, int rank_slot_base, int* route_order,
-                               int* tile_rank_counts, int64_t* copied_topk_idx, int* cumulative_expert_stats) {
+                               int* rank_prefix_matrix, int* slot_rel, int* rank_slot_idx, int rank_slot_base,
+                               int* route_order, int* tile_rank_counts, int64_t* copied_topk_idx,
+                               int* cumulative_expert_stats) {
   if (num_tokens < 0 || num_topk <= 0 || num_ranks <= 0 || num_experts <= 0 || expert_alignment < 1)
     return MI_EP_EINVAL;
   if (num_tokens_per_rank == nullptr || num_tokens_per_expert == nullptr) return MI_EP_EINVAL;
@@ -116,6 +117,8 @@ int mi_ep_host_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_
   int* d_off = expert_offsets != nullptr ? s.alloc<int>(static_cast<size_t>(num_experts) + 1) : nullptr;
   int* d_psum = psum_rank_rows != nullptr ? s.alloc<int>(num_ranks) : nullptr;
   int* d_prefix = channel_prefix_matrix != nullptr ? s.alloc<int>(rc) : nullptr;
+  const size_t rr = static_cast<size_t>(num_ranks) * num_ranks;
+  int* d_rank_prefix = rank_prefix_matrix != nullptr ? s.alloc<int>(rr) : nullptr;
   int* d_slot_rel = slot_rel != nullptr ? s.alloc<int>(tk) : nullptr;
   int* d_rank_slots = rank_slot_idx != nullptr ? s.alloc<int>(tk) : nullptr;
   int* d_order = route_order != nullptr ? s.alloc<int>(order_ints) : nullptr;
@@ -136,8 +139,8 @@ int mi_ep_host_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_
   int code = mi_ep_workspace_init(d_ws, workspace_bytes, nullptr);
   if (code == MI_EP_OK)
     code = mi_ep_dispatch_layout(d_topk, num_tokens, num_topk, num_ranks, num_experts, expert_alignment,
-                                 num_channels, d_rank, d_expert, d_flags, d_off, d_psum, d_prefix, d_slot_rel,
-                                 d_rank_slots, rank_slot_base, d_order, d_tile_ranks, d_copied, d_stats, d_ws,
+                                 num_channels, d_rank, d_expert, d_flags, d_off, d_psum, d_prefix, d_rank_prefix,
+                                 d_slot_rel, d_rank_slots, rank_slot_base, d_order, d_tile_ranks, d_copied, d_stats, d_ws,
                                  workspace_bytes, nullptr);
   if (code == MI_EP_OK) code = mi_ep_workspace_status(d_ws, nullptr);  // synchronises
   if (code != MI_EP_OK) return code;
@@ -147,6 +150,7 @@ int mi_ep_host_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_
   s.download(expert_offsets, d_off, static_cast<size_t>(num_experts) + 1);
   s.download(psum_rank_rows, d_psum, num_ranks);
   s.download(channel_prefix_matrix, d_prefix, rc);
+  s.download(rank_prefix_matrix, d_rank_prefix, rr);
   s.download(slot_rel, d_slot_rel, tk);
   s.download(rank_slot_idx, d_rank_slots, tk);
   s.download(route_order, d_order, order_ints);
@@ -200,8 +204,8 @@ int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* top
   int code = mi_ep_workspace_init(d_ws, workspace_bytes, nullptr);
   if (code == MI_EP_OK)
     code = mi_ep_dispatch_layout(d_topk, num_tokens, num_topk, num_ranks, num_experts, expert_alignment, 0,
-                                 d_rank, d_expert, d_flags, d_off, nullptr, nullptr, d_slot_rel, nullptr, 0,
-                                 d_order, nullptr, nullptr, nullptr, d_ws, workspace_bytes, nullptr);
+                                 d_rank, d_expert, d_flags, d_off, nullptr, nullptr, nullptr, d_slot_rel, nullptr,
+                                 0, d_order, nullptr, nullptr, nullptr, d_ws, workspace_bytes, nullptr);
   if (code == MI_EP_OK)
     code = mi_ep_dispatch(d_x, d_scales, d_topk, d_w, d_off, d_slot_rel, d_order, d_expert, num_tokens,
                           num_topk, num_experts, expert_alignment, row_bytes, num_scales, d_recv_x,
@@ -271,8 +275,8 @@ int mi_ep_host_dispatch_ranks(const void* x, const float* x_scales, const int64_
   int code = mi_ep_workspace_init(d_ws, workspace_bytes, nullptr);
   if (code == MI_EP_OK)
     code = mi_ep_dispatch_layout(d_topk, num_tokens, num_topk, num_ranks, num_experts, 1, 0, d_rank, d_expert,
-                                 d_flags, nullptr, nullptr, nullptr, nullptr, d_rank_slots, 0, nullptr, nullptr,
-                                 nullptr, nullptr, d_ws, workspace_bytes, nullptr);
+                                 d_flags, nullptr, nullptr, nullptr, nullptr, nullptr, d_rank_slots, 0, nullptr,
+                                 nullptr, nullptr, nullptr, d_ws, workspace_bytes, nullptr);
   if (code == MI_EP_OK)
     code = mi_ep_dispatch_ranks(d_x, d_scales, d_topk, d_w, d_rank_slots, 0, d_rank, nullptr, num_tokens,
                                 num_topk, num_ranks, num_experts, row_bytes, num_scales, source_token_base,

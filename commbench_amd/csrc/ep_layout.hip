@@ -500,19 +500,38 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
     }
   }
 
-  // ---- per-channel inclusive prefix: the tile holding a channel's end writes it
-  if (a.channel_prefix_matrix != nullptr) {
-    const int C = a.num_channels;
-    const int per_channel = (T + C - 1) / C;
-    for (int idx = tid; idx < C * R; idx += kLayoutThreads) {
-      const int c = idx / R, r = idx - c * R;
-      const long long s64 = static_cast<long long>(per_channel) * c;
+  // ---- per-channel and per-source-chunk inclusive prefixes: the tile holding a range's end
+  // writes it.  Ranges are the reference's get_channel_task_range (example047 .cu:73-79): range c
+  // of C covers [min(per * c, T), min(per * c + per, T)) with per = ceil(T / C).  The channel matrix
+  // is [rank, channel]; the rank prefix matrix takes the tokens as R such chunks, one per source rank,
+  // and is [source, rank] (rank_prefix_matrix_copy, example047 .cu:128-143,352-360).
+  if (a.channel_prefix_matrix != nullptr || a.rank_prefix_matrix != nullptr) {
+    // Tokens among the tile's first n that are flagged for rank r: whole waves from the per-wave
+    // counts, the rest from the flag words.
+    auto flagged_before = [&](const int r, const int n) -> int {
+      if (n >= kTileTokens) return col_total[E + r];
+      int cnt = 0;
+      for (int w = 0; w < (n >> 6); ++w) cnt += rank_wave[w * kMaxRanks + r];
+      for (int tl = n & ~(kWave - 1); tl < n; ++tl) cnt += static_cast<int>((tok_flags[tl] >> (8 * r)) & 1u);
+      return cnt;
+    };
+    const int C = a.channel_prefix_matrix != nullptr ? a.num_channels : 0;
+    const int chunks = a.rank_prefix_matrix != nullptr ? R : 0;
+    for (int idx = tid; idx < (C + chunks) * R; idx += kLayoutThreads) {
+      const int c_all = idx / R, r = idx - c_all * R;
+      const bool channel = c_all < C;
+      const int c = channel ? c_all : c_all - C;
+      const int ranges = channel ? C : R;
+      const int per_range = (T + ranges - 1) / ranges;
+      const long long s64 = static_cast<long long>(per_range) * c;
       const int start = s64 < T ? static_cast<int>(s64) : T;
-      const int end = (T - start < per_channel) ? T : start + per_channel;
+      const int end = (T - start < per_range) ? T : start + per_range;
       if (end > t0 && end <= t0 + kTileTokens) {
-        int cnt = 0;
-        for (int tl = 0; tl < end - t0; ++tl) cnt += static_cast<int>((tok_flags[tl] >> (8 * r)) & 1u);
-        a.channel_prefix_matrix[r * C + c] = col_excl[E + r] + cnt;
+        const int value = col_excl[E + r] + flagged_before(r, end - t0);
+        if (channel)
+          a.channel_prefix_matrix[r * C + c] = value;
+        else
+          a.rank_prefix_matrix[c * R + r] = value;
       }
     }
   }
@@ -561,13 +580,71 @@ __global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const L
   }
 }
 
-// Counts and flags only.  One token per thread, 1024 tokens per workgroup pass; totals are
-// accumulated with global atomics into zeroed outputs, or stored directly when one
-// workgroup covers every token.
+// Counts and flags only, up to 1024 tokens: one workgroup, one token per thread, one launch and
+// one barrier.  What bounds a call this small is its chain of latencies, so everything hangs off
+// the first load: a thread fetches its token's ids, the wave zeroes and fills its private row of
+// counters (equal experts found with ballots, the lowest lane of a group adds the group's size: no
+// atomics, no barrier before them), the token's flags go out from registers, and after the only
+// barrier thread e adds up column e of the waves' rows and stores the total.
+__global__ __launch_bounds__(kCountsThreads) void ep_layout_counts_small_kernel(
+    const int64_t* __restrict__ topk_idx, int* num_tokens_per_rank, int* num_tokens_per_expert,
+    uint8_t* is_token_in_rank, const int T, const int K, const int R, const int E,
+    const uint32_t inv_experts_per_rank, const int expert_bits) {
+  extern __shared__ int smem[];
+  const int tid = static_cast<int>(threadIdx.x);
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int waves = static_cast<int>(blockDim.x) >> 6;
+  int* rank_wave = smem;                                                          // [waves][kMaxRanks]
+  uint16_t* hist = reinterpret_cast<uint16_t*>(smem + waves * kMaxRanks);         // [waves][E]: a wave holds at most 64 * 8 routes
+  uint16_t* my_hist = hist + wave * E;
+
+  int64_t ids[kMaxTopk];
+#pragma unroll
+  for (int k = 0; k < kMaxTopk; ++k)
+    ids[k] = (k < K && tid < T) ? topk_idx[static_cast<size_t>(tid) * K + k] : -1;
+  for (int i = lane; i < E; i += kWave) my_hist[i] = 0;
+  __builtin_amdgcn_wave_barrier();
+
+  uint64_t flags = 0;
+#pragma unroll
+  for (int k = 0; k < kMaxTopk; ++k) {
+    if (k < K) {
+      const bool valid = ids[k] >= 0 && ids[k] < static_cast<int64_t>(E);
+      const int e = valid ? static_cast<int>(ids[k]) : 0;
+      const uint64_t same = match_expert(valid, e, expert_bits);
+      if (valid) {
+        // One writer per counter and instruction: the lowest lane of every group of equal experts.
+        if ((same & lanes_below(lane)) == 0) my_hist[e] = static_cast<uint16_t>(my_hist[e] + __popcll(same));
+        flags |= 1ull << (8 * ((static_cast<uint32_t>(e) * inv_experts_per_rank) >> 22));
+      }
+    }
+  }
+  if (tid < T) store_token_flags(is_token_in_rank, tid, R, flags);
+#pragma unroll
+  for (int r = 0; r < kMaxRanks; ++r) {
+    const uint64_t hit = __ballot(r < R && ((flags >> (8 * r)) & 1u) != 0);
+    if (lane == 0) rank_wave[wave * kMaxRanks + r] = __popcll(hit);
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += static_cast<int>(blockDim.x)) {
+    int total = 0;
+    for (int w = 0; w < waves; ++w) total += hist[w * E + e];
+    num_tokens_per_expert[e] = total;
+  }
+  if (tid < R) {
+    int total = 0;
+    for (int w = 0; w < waves; ++w) total += rank_wave[w * kMaxRanks + tid];
+    num_tokens_per_rank[tid] = total;
+  }
+}
+
+// Counts and flags only, more than 1024 tokens.  One token per thread, 1024 tokens per workgroup
+// pass; totals are accumulated with global atomics into zeroed outputs.
 __global__ __launch_bounds__(kCountsThreads) void ep_layout_counts_kernel(
     const int64_t* __restrict__ topk_idx, int* num_tokens_per_rank, int* num_tokens_per_expert,
     uint8_t* is_token_in_rank, int T, int K, int R, int E, int experts_per_rank, int expert_bits,
-    int num_tiles, int single_workgroup) {
+    int num_tiles) {
   extern __shared__ int smem[];
   int* hist = smem;                // [E]
   int* rank_cnt = hist + E;        // [kMaxRanks]
@@ -615,12 +692,6 @@ __global__ __launch_bounds__(kCountsThreads) void ep_layout_counts_kernel(
     __syncthreads();
   }
   __syncthreads();
-  if (single_workgroup) {
-    // The only workgroup has seen every token: plain stores, no zeroing pass needed.
-    for (int i = tid; i < E; i += kCountsThreads) num_tokens_per_expert[i] = hist[i];
-    if (tid < R) num_tokens_per_rank[tid] = rank_cnt[tid];
-    return;
-  }
   for (int i = tid; i < E; i += kCountsThreads)
     if (hist[i] != 0) atomicAdd(&num_tokens_per_expert[i], hist[i]);
   if (tid < R && rank_cnt[tid] != 0) atomicAdd(&num_tokens_per_rank[tid], rank_cnt[tid]);
@@ -665,26 +736,32 @@ hipError_t launch_layout_counts(const int64_t* topk_idx, int* num_tokens_per_ran
                                 int* num_tokens_per_expert, uint8_t* is_token_in_rank,
                                 int num_tokens, int num_topk, int num_ranks, int num_experts,
                                 hipStream_t stream) {
-  const int num_tiles = (num_tokens + kCountsThreads - 1) / kCountsThreads;
-  // Up to 1024 tokens one workgroup sees everything and stores the totals itself: one
-  // launch instead of zero + accumulate, which is what matters at these sizes.
-  const bool single = num_tiles == 1;
-  if (!single) {
-    const int n = num_experts > num_ranks ? num_experts : num_ranks;
-    hipLaunchKernelGGL(ep_zero_counts_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
-                       num_tokens_per_expert, num_experts, num_tokens_per_rank, num_ranks);
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess || num_tokens == 0) return err;
-  }
   int expert_bits = 1;
   while ((1 << expert_bits) < num_experts) ++expert_bits;
-  const int grid = single ? 1 : (num_tiles < 1024 ? num_tiles : 1024);
+  const int experts_per_rank = num_experts / num_ranks;
+  if (num_tokens <= kCountsThreads) {
+    // One workgroup sees everything and stores the totals itself: one launch instead of zero +
+    // accumulate, which is what matters at these sizes (no tokens: one wave stores the zeros).
+    const int waves = num_tokens > 0 ? (num_tokens + kWave - 1) / kWave : 1;
+    const size_t lds = static_cast<size_t>(waves) * (sizeof(int) * kMaxRanks + sizeof(uint16_t) * num_experts);
+    const uint32_t inv_experts_per_rank = ((1u << 22) + experts_per_rank - 1) / experts_per_rank;
+    hipLaunchKernelGGL(ep_layout_counts_small_kernel, dim3(1), dim3(waves * kWave), lds, stream, topk_idx,
+                       num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, num_tokens, num_topk,
+                       num_ranks, num_experts, inv_experts_per_rank, expert_bits);
+    return hipGetLastError();
+  }
+  const int num_tiles = (num_tokens + kCountsThreads - 1) / kCountsThreads;
+  const int n = num_experts > num_ranks ? num_experts : num_ranks;
+  hipLaunchKernelGGL(ep_zero_counts_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
+                     num_tokens_per_expert, num_experts, num_tokens_per_rank, num_ranks);
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  const int grid = num_tiles < 1024 ? num_tiles : 1024;
   const size_t lds = sizeof(int) * (num_experts + kMaxRanks + (num_experts & 1)) +
                      sizeof(uint64_t) * kCountsThreads;
   hipLaunchKernelGGL(ep_layout_counts_kernel, dim3(grid), dim3(kCountsThreads), lds, stream, topk_idx,
                      num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, num_tokens, num_topk,
-                     num_ranks, num_experts, num_experts / num_ranks, expert_bits, num_tiles,
-                     single ? 1 : 0);
+                     num_ranks, num_experts, experts_per_rank, expert_bits, num_tiles);
   return hipGetLastError();
 }
 

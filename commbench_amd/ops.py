@@ -91,6 +91,7 @@ class DispatchHandle:
     expert_offsets: torch.Tensor           # int32[E + 1], exclusive over aligned counts
     psum_rank_rows: torch.Tensor           # int32[R], inclusive rows per partition
     channel_prefix_matrix: Optional[torch.Tensor]  # int32[R, C]
+    rank_prefix_matrix_: torch.Tensor      # int32[R, R], [source chunk, destination rank]
     slot_rel: torch.Tensor                 # int32[T, K]
     rank_slot_idx: Optional[torch.Tensor] = None   # int32[T, K], the prologue's dst_buffer_slot_idx
     route_order: Optional[torch.Tensor] = None     # int32[tiles * 256 * K, 4], routes in destination order
@@ -109,10 +110,8 @@ class DispatchHandle:
         """int32[src, dst]: tokens of source chunks 0..src flagged for rank dst, the tokens taken as
         num_ranks equal contiguous chunks (ceil(T / R) tokens each): the notify example's
         rank_prefix_matrix (example047 .cu:128-143,352-360) with chunks of this GPU's tokens standing
-        for source ranks.  Needs a layout that ran with num_channels == num_ranks."""
-        _require(self.channel_prefix_matrix is not None and self.channel_prefix_matrix.shape[1] == self.num_ranks,
-                 "rank_prefix_matrix needs a layout with num_channels == num_ranks")
-        return self.channel_prefix_matrix.t().contiguous()
+        for source ranks.  Written by the layout launch itself, whatever its num_channels."""
+        return self.rank_prefix_matrix_
 
 
 class Buffer:
@@ -181,6 +180,7 @@ class Buffer:
             psum_rank_rows=torch.empty(R, dtype=torch.int32, device=dev),
             channel_prefix_matrix=(torch.empty((R, num_channels), dtype=torch.int32, device=dev)
                                    if num_channels > 0 else None),
+            rank_prefix_matrix_=torch.empty((R, R), dtype=torch.int32, device=dev),
             slot_rel=torch.empty((T, K), dtype=torch.int32, device=dev),
             rank_slot_idx=(torch.empty((T, K), dtype=torch.int32, device=dev)
                            if rank_slot_base is not None else None),
@@ -201,10 +201,10 @@ class Buffer:
             _ptr(topk_idx), T, K, R, E, expert_alignment, num_channels,
             _ptr(h.num_tokens_per_rank), _ptr(h.num_tokens_per_expert), _ptr(h.is_token_in_rank),
             _ptr(h.expert_offsets), _ptr(h.psum_rank_rows), _ptr(h.channel_prefix_matrix),
-            _ptr(h.slot_rel), _ptr(h.rank_slot_idx), rank_slot_base or 0, _ptr(h.route_order),
-            _ptr(h.tile_rank_counts), _ptr(h.copied_topk_idx), _ptr(cumulative_expert_stats),
-            _ptr(self.workspace),
-            self.workspace.numel(), _stream()), "mi_ep_dispatch_layout")
+            _ptr(h.rank_prefix_matrix_), _ptr(h.slot_rel), _ptr(h.rank_slot_idx), rank_slot_base or 0,
+            _ptr(h.route_order), _ptr(h.tile_rank_counts), _ptr(h.copied_topk_idx),
+            _ptr(cumulative_expert_stats), _ptr(self.workspace), self.workspace.numel(), _stream()),
+            "mi_ep_dispatch_layout")
         return h
 
     def dispatch(self, x: torch.Tensor, scales: Optional[torch.Tensor], topk_idx: torch.Tensor,
@@ -562,6 +562,7 @@ def host_dispatch_layout(topk_idx, num_experts: int, num_ranks: int, expert_alig
         is_token_in_rank=np.empty((T, R), dtype=np.bool_), expert_offsets=np.empty(E + 1, dtype=np.int32),
         psum_rank_rows=np.empty(R, dtype=np.int32),
         channel_prefix_matrix=np.empty((R, num_channels), dtype=np.int32) if num_channels > 0 else None,
+        rank_prefix_matrix=np.empty((R, R), dtype=np.int32),
         slot_rel=np.empty((T, K), dtype=np.int32), rank_slot_idx=np.empty((T, K), dtype=np.int32),
         route_order=np.empty((order_rows, 4), dtype=np.int32),
         tile_rank_counts=np.empty(((T + 255) // 256, R), dtype=np.int32),
@@ -569,7 +570,8 @@ def host_dispatch_layout(topk_idx, num_experts: int, num_ranks: int, expert_alig
     _lib.check(_lib.load().mi_ep_host_dispatch_layout(
         _np_ptr(topk_idx), T, K, R, E, expert_alignment, num_channels, _np_ptr(out["num_tokens_per_rank"]),
         _np_ptr(out["num_tokens_per_expert"]), _np_ptr(out["is_token_in_rank"]), _np_ptr(out["expert_offsets"]),
-        _np_ptr(out["psum_rank_rows"]), _np_ptr(out["channel_prefix_matrix"]), _np_ptr(out["slot_rel"]),
+        _np_ptr(out["psum_rank_rows"]), _np_ptr(out["channel_prefix_matrix"]),
+        _np_ptr(out["rank_prefix_matrix"]), _np_ptr(out["slot_rel"]),
         _np_ptr(out["rank_slot_idx"]), rank_slot_base, _np_ptr(out["route_order"]),
         _np_ptr(out["tile_rank_counts"]), _np_ptr(out["copied_topk_idx"]), _np_ptr(cumulative_expert_stats)),
         "mi_ep_host_dispatch_layout")

@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define MI_EP_ABI_VERSION 2
+#define MI_EP_ABI_VERSION 3
 
 #define MI_EP_OK 0
 #define MI_EP_EINVAL (-22)    /* argument out of range or NULL where required */
@@ -63,7 +63,12 @@ int mi_ep_get_dispatch_layout(const int64_t* topk_idx, int* num_tokens_per_rank,
  * It must be 8-byte aligned; with 16-byte alignment (any hipMalloc result) grids
  * of up to a few dozen tiles scan their tiles' totals with wide loads, which is
  * about 2 us faster per launch.
+ * The three calls that take a workspace pointer below (init, status, set_wait_limit) also accept
+ * MI_EP_STATIC_SCRATCH: the library's own scratch of mi_ep_dispatch_layout_static on the device
+ * `stream` belongs to (workspace_bytes is ignored then).  That scratch starts initialised;
+ * initialising it again clears a reported time-out.
  */
+#define MI_EP_STATIC_SCRATCH ((void*)(size_t)256)
 size_t mi_ep_workspace_bytes(int num_tokens, int num_topk, int num_experts, int num_ranks);
 int mi_ep_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 /* Synchronises `stream`, then reports MI_EP_ETIMEDOUT if any launch on this
@@ -107,6 +112,14 @@ int mi_ep_dispatch_schedule_for(int num_tokens, int num_topk, int num_experts, i
  *   psum_rank_rows      int32[num_ranks]; inclusive rows of partitions 0..r
  *   channel_prefix_matrix int32[num_ranks, num_channels]; tokens flagged for rank r in
  *                       token tiles 0..c (tile bounds as get_channel_task_range, :73-79)
+ *   rank_prefix_matrix  int32[num_ranks, num_ranks], source-major: [src, dst] = tokens of source
+ *                       chunks 0..src flagged for rank dst, the tokens taken as num_ranks contiguous
+ *                       chunks of ceil(num_tokens / num_ranks) (the same range rule, :73-79), one per
+ *                       source rank: rank_prefix_matrix_copy of notify_dispatch
+ *                       (empty_deepep_intranode_notify_dispatch.cu:112-143, checked at :352-384),
+ *                       which the reference gathers from R GPUs and this GPU's partitions provide
+ *                       in the same launch as the channel matrix; row num_ranks - 1 equals
+ *                       num_tokens_per_rank
  *   slot_rel            int32[num_tokens, num_topk]; position of route (t,k) inside its
  *                       expert segment in (token, slot) order, -1 for non-routes
  *   rank_slot_idx       int32[num_tokens, num_topk]; the prologue's own output format
@@ -137,8 +150,8 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
                           int num_experts, int expert_alignment, int num_channels,
                           int* num_tokens_per_rank, int* num_tokens_per_expert,
                           bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
-                          int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
-                          int rank_slot_base, int* route_order, int* tile_rank_counts,
+                          int* channel_prefix_matrix, int* rank_prefix_matrix, int* slot_rel,
+                          int* rank_slot_idx, int rank_slot_base, int* route_order, int* tile_rank_counts,
                           int64_t* copied_topk_idx, int* cumulative_expert_stats, void* workspace,
                           size_t workspace_bytes, void* stream);
 /*
@@ -153,22 +166,28 @@ int mi_ep_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
  *            MI_EP_E2BIG and launches nothing.
  *   timeout_report  NULL, or one int32 of device memory that the caller has set to 0: receives
  *            MI_EP_ETIMEDOUT if a bounded device-side wait of this launch expires (the outputs are
- *            then unspecified); never written otherwise.
+ *            then unspecified); never written otherwise.  With or without it,
+ *            mi_ep_workspace_status(MI_EP_STATIC_SCRATCH, stream) reports an expired wait since the
+ *            scratch was last initialised, mi_ep_workspace_set_wait_limit(MI_EP_STATIC_SCRATCH, ...)
+ *            bounds the waits and mi_ep_workspace_init(MI_EP_STATIC_SCRATCH, 0, stream) clears the
+ *            report.
  * Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
  * streams, two threads) race and give unspecified results; calls ordered on one stream, or
- * otherwise serialised, are safe back to back whatever their shapes.  The first call on a device
- * resolves the array's address (hipGetSymbolAddress, which may load the code object): make it
- * outside graph capture.  Calls hipMalloc / hipFree never.
+ * otherwise serialised, are safe back to back whatever their shapes.  The array used is the one
+ * of the device `stream` belongs to (of the current device for NULL), whatever device is current.
+ * The first call on a device resolves the array's address (hipGetSymbolAddress, which may load the
+ * code object): make it outside graph capture; the address does not outlive a hipDeviceReset.
+ * Calls hipMalloc / hipFree never.
  */
 #define MI_EP_STATIC_LAYOUT_STATUS_WORDS 262144
 int mi_ep_dispatch_layout_static(const int64_t* topk_idx, int num_tokens, int num_topk, int num_ranks,
                                  int num_experts, int expert_alignment, int num_channels,
                                  int* num_tokens_per_rank, int* num_tokens_per_expert,
                                  bool* is_token_in_rank, int* expert_offsets, int* psum_rank_rows,
-                                 int* channel_prefix_matrix, int* slot_rel, int* rank_slot_idx,
-                                 int rank_slot_base, int* route_order, int* tile_rank_counts,
-                                 int64_t* copied_topk_idx, int* cumulative_expert_stats,
-                                 int* timeout_report, void* stream);
+                                 int* channel_prefix_matrix, int* rank_prefix_matrix, int* slot_rel,
+                                 int* rank_slot_idx, int rank_slot_base, int* route_order,
+                                 int* tile_rank_counts, int64_t* copied_topk_idx,
+                                 int* cumulative_expert_stats, int* timeout_report, void* stream);
 /* Bytes of route_order for this shape. */
 size_t mi_ep_route_order_bytes(int num_tokens, int num_topk);
 
@@ -396,8 +415,9 @@ int mi_ep_host_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_
                                int num_experts, int expert_alignment, int num_channels,
                                int* num_tokens_per_rank, int* num_tokens_per_expert, bool* is_token_in_rank,
                                int* expert_offsets, int* psum_rank_rows, int* channel_prefix_matrix,
-                               int* slot_rel, int* rank_slot_idx, int rank_slot_base, int* route_order,
-                               int* tile_rank_counts, int64_t* copied_topk_idx, int* cumulative_expert_stats);
+                               int* rank_prefix_matrix, int* slot_rel, int* rank_slot_idx, int rank_slot_base,
+                               int* route_order, int* tile_rank_counts, int64_t* copied_topk_idx,
+                               int* cumulative_expert_stats);
 int mi_ep_host_dispatch(const void* x, const float* x_scales, const int64_t* topk_idx,
                         const float* topk_weights, int num_tokens, int num_topk, int num_ranks,
                         int num_experts, int expert_alignment, int row_bytes, int num_scales,

@@ -92,6 +92,7 @@ struct DispatchHandle {
   int* expert_offsets = nullptr;         // [E + 1]
   int* psum_rank_rows = nullptr;         // [R]
   int* channel_prefix_matrix = nullptr;  // [R, C] (C = num_channels of the buffer, may be 0)
+  int* rank_prefix_matrix = nullptr;     // [R, R] source-major, the notify example's rank_prefix_matrix_copy
   int* slot_rel = nullptr;               // [T, K]
   int* rank_slot_idx = nullptr;          // [T, K] the deterministic prologue's table (base 0)
   int* route_order = nullptr;            // [tiles * 256 * K, 4] routes in destination order
@@ -132,6 +133,7 @@ class ExpertParallelBuffer {
     MI_EP_HIP_CHECK(hipMalloc(&h_.psum_rank_rows, sizeof(int) * num_ranks));
     if (num_channels > 0)
       MI_EP_HIP_CHECK(hipMalloc(&h_.channel_prefix_matrix, sizeof(int) * num_ranks * num_channels));
+    MI_EP_HIP_CHECK(hipMalloc(&h_.rank_prefix_matrix, sizeof(int) * num_ranks * num_ranks));
     MI_EP_HIP_CHECK(hipMalloc(&h_.slot_rel, sizeof(int) * (tk + 1)));
     MI_EP_HIP_CHECK(hipMalloc(&h_.rank_slot_idx, sizeof(int) * (tk + 1)));
     MI_EP_HIP_CHECK(hipMalloc(&h_.rank_row_map, sizeof(int) * (tk + 1)));
@@ -153,7 +155,7 @@ class ExpertParallelBuffer {
                      h_.expert_offsets, h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel,
                      h_.rank_slot_idx, h_.rank_row_map, h_.rank_combine_map, h_.psum_rank_tokens,
                      h_.route_order, h_.slot_map, h_.recv_src_map, h_.recv_topk_idx, h_.recv_topk_weights,
-                     h_.tile_rank_counts, h_.copied_topk_idx};
+                     h_.tile_rank_counts, h_.copied_topk_idx, h_.rank_prefix_matrix};
     for (void* p : owned)
       if (p != nullptr) (void)hipFree(p);
   }
@@ -167,7 +169,8 @@ class ExpertParallelBuffer {
   // its counts (the reference's cumulative_local_expert_recv_stats); nullptr switches it off.
   void set_cumulative_expert_stats(int* d_stats) { cumulative_expert_stats_ = d_stats; }
 
-  // Fused layout: counts, flags, offsets, per-route segment positions (and channel prefixes).
+  // Fused layout: counts, flags, offsets, per-route segment positions, the rank prefix matrix (and
+  // channel prefixes when the buffer has channels).
   // with_rank_slots also fills rank_slot_idx, the deterministic prologue's per-rank slot table.
   const DispatchHandle& get_dispatch_layout(const TopkIdx* d_topk_idx, int num_tokens, hipStream_t stream = 0,
                                             bool with_rank_slots = false) {
@@ -176,7 +179,7 @@ class ExpertParallelBuffer {
     MI_EP_CHECK(mi_ep_dispatch_layout(d_topk_idx, num_tokens, num_topk_, num_ranks_, num_experts_,
                                       h_.expert_alignment, num_channels_, h_.num_tokens_per_rank,
                                       h_.num_tokens_per_expert, h_.is_token_in_rank, h_.expert_offsets,
-                                      h_.psum_rank_rows, h_.channel_prefix_matrix, h_.slot_rel,
+                                      h_.psum_rank_rows, h_.channel_prefix_matrix, h_.rank_prefix_matrix, h_.slot_rel,
                                       with_rank_slots ? h_.rank_slot_idx : nullptr, /*rank_slot_base=*/0, h_.route_order,
                                       h_.tile_rank_counts, h_.copied_topk_idx, cumulative_expert_stats_,
                                       workspace_, workspace_bytes_, stream));

@@ -24,6 +24,7 @@ int ep_oracle_layout(const int64_t*, int, int, int, int, int*, int*, uint8_t*);
 int ep_oracle_expert_offsets(const int*, int, int, int, int*, int*);
 int ep_oracle_slot_maps(const int64_t*, int, int, int, const int*, int*, int*, int*, int*, int*);
 int ep_oracle_channel_prefix(const uint8_t*, int, int, int, int*);
+void ep_oracle_rank_prefix(const int*, int, int*);
 int ep_oracle_permute(const void*, int, const float*, int, const int64_t*, const float*, int, const int*,
                       const int*, int, void*, float*, int64_t*, float*, int);
 int ep_oracle_permute_ranks(const void*, int, const float*, int, const int64_t*, const float*, int, int, int, int, int,
@@ -150,25 +151,39 @@ bool check_fused_surface(const Case& c, int align, int channels) {
   return ok;
 }
 
-// The notify example's inputs (example047 .cu:189-193,437-447) for source rank 0: two
-// destinations per token, one expert per rank; C = min(16, max(4, 2R)).
+// The notify example's inputs (example047 .cu:189-193,437-447): the batches of all R source ranks,
+// `tokens` each, laid end to end (two destinations per token, one expert per rank), so that the R
+// source chunks of the launch are exactly the R ranks' batches; C = min(16, max(4, 2R)).  One launch
+// must give the harness's expected rank prefix matrix (.cu:352-360) and the per-channel prefix of
+// the whole batch (.cu:386-428).
 bool check_notify_case(int tokens, int ranks) {
-  Case c{tokens, std::min(2, ranks), ranks, ranks, kSpread};
-  std::vector<TopkIdx> idx(static_cast<size_t>(tokens) * c.topk);
-  for (int t = 0; t < tokens; ++t)
-    for (int s = 0; s < c.topk; ++s) idx[static_cast<size_t>(t) * c.topk + s] = (t + s) % ranks;
+  const int total = tokens * ranks;
+  Case c{total, std::min(2, ranks), ranks, ranks, kSpread};
+  std::vector<TopkIdx> idx(static_cast<size_t>(total) * c.topk);
+  std::vector<int> counts(static_cast<size_t>(ranks) * ranks, 0);
+  for (int src = 0; src < ranks; ++src) {
+    const int stride = ranks > 1 ? src % (ranks - 1) + 1 : 0;
+    for (int t = 0; t < tokens; ++t)
+      for (int s = 0; s < c.topk; ++s) {
+        const int dst = (t + src + s * stride) % ranks;
+        idx[(static_cast<size_t>(src) * tokens + t) * c.topk + s] = dst;
+        ++counts[static_cast<size_t>(src) * ranks + dst];  // distinct per token: stride is in [1, R)
+      }
+  }
   const int channels = std::min(16, std::max(4, 2 * ranks));
   const HostLayout ref = host_layout(c, idx, 1);
-  std::vector<int> want(static_cast<size_t>(ranks) * channels);
-  ep_oracle_channel_prefix(ref.flags.data(), tokens, ranks, channels, want.data());
+  std::vector<int> want(static_cast<size_t>(ranks) * channels), want_rank(counts.size());
+  ep_oracle_channel_prefix(ref.flags.data(), total, ranks, channels, want.data());
+  ep_oracle_rank_prefix(counts.data(), ranks, want_rank.data());
   DeviceArray<TopkIdx> d_idx(idx.size());
   d_idx.upload(idx);
-  mi_ep::ExpertParallelBuffer buf(tokens, c.topk, ranks, ranks, 1, channels);
-  const mi_ep::DispatchHandle& h = buf.get_dispatch_layout(d_idx.p, tokens);
+  mi_ep::ExpertParallelBuffer buf(total, c.topk, ranks, ranks, 1, channels);
+  const mi_ep::DispatchHandle& h = buf.get_dispatch_layout(d_idx.p, total);
   buf.check_status();
-  std::vector<int> got(want.size());
+  std::vector<int> got(want.size()), got_rank(want_rank.size());
   MI_EP_HIP_CHECK(hipMemcpy(got.data(), h.channel_prefix_matrix, got.size() * sizeof(int), hipMemcpyDeviceToHost));
-  return got == want;
+  MI_EP_HIP_CHECK(hipMemcpy(got_rank.data(), h.rank_prefix_matrix, got_rank.size() * sizeof(int), hipMemcpyDeviceToHost));
+  return got == want && got_rank == want_rank;
 }
 
 // Dispatch -> identity experts -> weighted combine on a small bf16 case, against the checker.
@@ -307,6 +322,18 @@ MetricRow time_launches(const std::string& surface, const Case& c, Launch launch
   row.latency_us = static_cast<double>(ms) * 1000.0 / bench_iters;
   row.mtokens_per_s = row.latency_us > 0.0 ? c.tokens / row.latency_us : 0.0;
   return row;
+}
+
+// What one launch costs when the kernel does nothing: one wave that returns at once, timed like
+// every other row (20 + 100 back-to-back launches between two events).  No layout call at a small
+// batch can be faster than this.
+__global__ void ep_selftest_empty_kernel() {}
+
+void benchmark_launch_floor(std::vector<MetricRow>* rows) {
+  MetricRow row = time_launches("launch_floor", Case{0, 1, 1, 1, kSpread},
+                                [] { hipLaunchKernelGGL(ep_selftest_empty_kernel, dim3(1), dim3(64), 0, nullptr); });
+  MI_EP_HIP_CHECK(hipGetLastError());
+  rows->push_back(row);
 }
 
 void benchmark_case(const Case& c, std::vector<MetricRow>* rows) {
@@ -452,6 +479,7 @@ int main(int argc, char** argv) {
 
   std::vector<MetricRow> rows;
   if (!skip_bench) {
+    benchmark_launch_floor(&rows);
     for (int tokens : {1024, 4096, 16384, 65536}) benchmark_case({tokens, 2, 8, 32, kSpread}, &rows);
     benchmark_case({65536, 4, 8, 32, kRankSweep}, &rows);
     benchmark_case({65536, 8, 8, 32, kSameRank}, &rows);

@@ -47,6 +47,19 @@ def run_fused_layout(buf: ops.Buffer, topk_idx_np, expert_alignment=1, num_chann
     return topk, h
 
 
+def source_chunk_counts(flags: np.ndarray, num_ranks: int) -> np.ndarray:
+    """int32[src, dst]: tokens of source chunk src flagged for rank dst, the tokens taken as num_ranks
+    contiguous chunks of ceil(T / R) (the notify example's range rule, example047 .cu:73-79); input
+    of oracle.rank_prefix."""
+    T = flags.shape[0]
+    per_chunk = -(-T // num_ranks) if T else 0
+    counts = np.zeros((num_ranks, num_ranks), dtype=np.int32)
+    for src in range(num_ranks):
+        start = min(per_chunk * src, T)
+        counts[src] = flags[start:min(start + per_chunk, T)].sum(axis=0)
+    return counts
+
+
 def check_layout_against_oracle(oracle, h, topk_np, R, E, align=1, channels=0):
     per_rank, per_expert, flags = oracle.layout(topk_np, R, E)
     off, psum = oracle.expert_offsets(per_expert, R, align)
@@ -69,5 +82,7 @@ def check_layout_against_oracle(oracle, h, topk_np, R, E, align=1, channels=0):
     if channels:
         np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy(),
                                       oracle.channel_prefix(flags, channels))
+    np.testing.assert_array_equal(h.rank_prefix_matrix().cpu().numpy(),
+                                  oracle.rank_prefix(source_chunk_counts(flags, R)))
     return dict(per_rank=per_rank, per_expert=per_expert, flags=flags, off=off, psum=psum,
                 slot_rel=slot_rel, slot_map=slot_map, src_map=src_map, src_k=src_k)

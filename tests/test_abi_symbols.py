@@ -61,7 +61,7 @@ def test_host_only_entry_points():
     """Calls that touch no device: version, error strings, workspace sizing, argument checks."""
     from commbench_amd import _lib
     lib = _lib.load()
-    assert lib.mi_ep_abi_version() == 2
+    assert lib.mi_ep_abi_version() == 3
     assert _lib.strerror(0) == "ok"
     assert _lib.strerror(-22) == "invalid argument"
     assert _lib.strerror(-28) == "workspace too small"
@@ -100,8 +100,8 @@ def test_host_only_entry_points():
     assert lib.mi_ep_dispatch_cached(None, None, None, 4, 4, 24, 0, None, None, None, 0, None) == -22
     assert lib.mi_ep_dispatch(None, None, None, None, None, None, None, None, 4, 2, 8, 1, 32, 0,
                               None, None, None, None, None, None, 0, 8, None) == -22   # null tables (and an unknown flag)
-    assert lib.mi_ep_host_dispatch_layout(None, 4, 2, 2, 8, 0, 0, None, None, None, None, None, None, None, None, 0,
-                                          None, None, None, None) == -22                # alignment 0
+    assert lib.mi_ep_host_dispatch_layout(None, 4, 2, 2, 8, 0, 0, None, None, None, None, None, None, None, None,
+                                          None, 0, None, None, None, None) == -22       # alignment 0
     assert lib.mi_ep_host_get_dispatch_layout(None, None, None, None, None, 4, 2, 2, 8) == -22
     assert lib.mi_ep_host_dispatch(None, None, None, None, 4, 2, 2, 8, 1, 24, 0, None, None, None, None,
                                    None, None, None, None, None, None, 0) == -22
@@ -116,11 +116,11 @@ def test_host_only_entry_points():
     assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 2, 9, 18, None) == -22
     assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 9, 2, 8, None) == -22
     assert lib.mi_ep_get_dispatch_layout(None, None, None, None, None, 4, 2, 3, 8, None) == -22
-    assert lib.mi_ep_dispatch_layout(None, 4, 2, 2, 8, 0, 0, None, None, None, None, None, None,
+    assert lib.mi_ep_dispatch_layout(None, 4, 2, 2, 8, 0, 0, None, None, None, None, None, None, None,
                                      None, None, 0, None, None, None, None, None, 0, None) == -22     # alignment 0
-    assert lib.mi_ep_dispatch_layout_static(None, 4, 2, 2, 8, 0, 0, None, None, None, None, None, None,
+    assert lib.mi_ep_dispatch_layout_static(None, 4, 2, 2, 8, 0, 0, None, None, None, None, None, None, None,
                                             None, None, 0, None, None, None, None, None, None) == -22  # alignment 0
-    assert lib.mi_ep_dispatch_layout_static(None, 1 << 20, 2, 8, 1024, 1, 0, None, None, None, None, None, None,
+    assert lib.mi_ep_dispatch_layout_static(None, 1 << 20, 2, 8, 1024, 1, 0, None, None, None, None, None, None, None,
                                             None, None, 0, None, None, None, None, None, None) == -7   # beyond the scratch
     assert lib.mi_ep_workspace_set_wait_limit(None, 1, None) == -22
     assert lib.mi_ep_combine(None, 0, None, None, None, None, None, None, 4, 2, 12, None, None, None, 0, None) == -22

@@ -387,9 +387,10 @@ def test_cached_pull_dispatch_and_pull_indices(oracle, payload):
 @pytest.mark.parametrize("shape", [(4096, 8), (4097, 8), (7, 2), (1000, 4), (333, 8), (5, 8)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_rank_prefix_matrix_from_channel_prefix(oracle, shape):
-    """One channel per source chunk: channel_prefix_matrix[dst, src] is the notify example's
-    rank_prefix_matrix[src, dst] (example047 .cu:352-360) for R contiguous source chunks of
-    ceil(T / R) tokens (its get_channel_task_range, .cu:73-79), ragged and empty chunks included."""
+    """The launch's rank_prefix_matrix[src, dst] is the notify example's (example047 .cu:352-360) for
+    R contiguous source chunks of ceil(T / R) tokens (its get_channel_task_range, .cu:73-79), ragged
+    and empty chunks included; with one channel per source chunk it is also the transposed channel
+    matrix of the same launch."""
     T, R = shape
     print(f"shape {shape}", flush=True)
     rng = np.random.default_rng(5 + T)
@@ -400,12 +401,9 @@ def test_rank_prefix_matrix_from_channel_prefix(oracle, shape):
     h = buf.dispatch_layout(torch.from_numpy(topk_np).to(gu.DEV), num_channels=R)
     torch.cuda.synchronize()
     _, _, flags = oracle.layout(topk_np, R, E)
-    per_chunk = -(-T // R)
-    counts = np.zeros((R, R), dtype=np.int32)
-    for src in range(R):
-        start = min(per_chunk * src, T)
-        counts[src] = flags[start:min(start + per_chunk, T)].sum(axis=0)
+    counts = gu.source_chunk_counts(flags, R)
     np.testing.assert_array_equal(h.rank_prefix_matrix().cpu().numpy(), oracle.rank_prefix(counts))
+    np.testing.assert_array_equal(h.rank_prefix_matrix().cpu().numpy(), h.channel_prefix_matrix.t().cpu().numpy())
     assert (h.rank_prefix_matrix()[-1].cpu().numpy() == h.num_tokens_per_rank.cpu().numpy()).all()
 
 

@@ -47,7 +47,7 @@ def test_graph_replays_match_eager(oracle, schedule):
     def step(stream):
         _lib.check(lib.mi_ep_dispatch_layout(
             topk.data_ptr(), T, K, R, E, 1, 0, per_rank.data_ptr(), per_expert.data_ptr(),
-            in_rank.data_ptr(), off.data_ptr(), psum.data_ptr(), None, slot_rel.data_ptr(), None, 0,
+            in_rank.data_ptr(), off.data_ptr(), psum.data_ptr(), None, None, slot_rel.data_ptr(), None, 0,
             route_order.data_ptr(), None, None, None, ws.data_ptr(), ws_bytes, stream), "layout")
         _lib.check(lib.mi_ep_dispatch(
             x.data_ptr(), None, topk.data_ptr(), w.data_ptr(), off.data_ptr(), slot_rel.data_ptr(),

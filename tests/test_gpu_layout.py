@@ -27,6 +27,30 @@ def test_get_dispatch_layout_reference_cases(oracle, case):
     np.testing.assert_array_equal(flags.cpu().numpy().view(np.uint8), w_flags)
 
 
+@pytest.mark.parametrize("shape", [
+    (1, 1, 1, 1), (1, 8, 8, 1024), (63, 3, 1, 5), (64, 8, 8, 8), (65, 2, 2, 6), (1000, 7, 4, 1024),
+    (1024, 8, 8, 256), (1025, 8, 8, 256), (5000, 5, 8, 1024)], ids=lambda s: "x".join(map(str, s)))
+def test_get_dispatch_layout_ragged_shapes(oracle, shape):
+    """Both forms of the counts-only layout (one workgroup up to 1024 tokens, many beyond) on ragged
+    token counts, every expert count's edge, masked, duplicated and out-of-range ids."""
+    T, K, R, E = shape
+    print(f"shape {shape}", flush=True)
+    rng = np.random.default_rng(T * 7 + E)
+    topk_np = rng.integers(-2, E + 2, size=(T, K)).astype(np.int64)
+    per_rank, per_expert, flags = ops.get_dispatch_layout(torch.from_numpy(topk_np).to(gu.DEV), E, R)
+    torch.cuda.synchronize()
+    w_rank, w_expert, w_flags = oracle.layout(topk_np, R, E)
+    np.testing.assert_array_equal(per_rank.cpu().numpy(), w_rank)
+    np.testing.assert_array_equal(per_expert.cpu().numpy(), w_expert)
+    np.testing.assert_array_equal(flags.cpu().numpy().view(np.uint8), w_flags)
+
+
+def test_get_dispatch_layout_without_tokens():
+    per_rank, per_expert, flags = ops.get_dispatch_layout(torch.zeros((0, 4), dtype=torch.int64, device=gu.DEV), 64, 8)
+    torch.cuda.synchronize()
+    assert not per_rank.cpu().numpy().any() and not per_expert.cpu().numpy().any() and flags.shape == (0, 8)
+
+
 def test_get_dispatch_layout_overwrites_its_outputs(oracle):
     """The reference's benchmark relaunches without re-zeroing (example042 .cu:313-329)."""
     from commbench_amd import _lib
@@ -165,17 +189,47 @@ def test_workspace_alternates_between_gathered_and_walked_scans(oracle):
         gu.check_layout_against_oracle(oracle, h, topk_np, R, E, 4, 8)
 
 
+def notify_topk(T, R, src_rank):
+    """Routing that reproduces the notify example's flags for one source rank (example047
+    .cu:189-193,437-447) with one expert per rank: slot s of token t goes to routeDst(src_rank, t, s)."""
+    t = np.arange(T)
+    stride = (src_rank % (R - 1)) + 1
+    return np.stack([(t + src_rank) % R, (t + src_rank + stride) % R], axis=1).astype(np.int64)
+
+
 @pytest.mark.parametrize("T", [7, 4096, 4097])
 @pytest.mark.parametrize("R", [2, 4, 8])
 def test_channel_prefix_reference_notify_cases(oracle, T, R):
-    """The reference's notify inputs (example047 .cu:599-610): two destinations per token."""
+    """The reference's notify inputs (example047 .cu:599-610), every source rank's batch in turn: two
+    destinations per token, C = min(16, max(4, 2R)) channels."""
     C = wl.reference_notify_channels(R)
-    flags = wl.reference_notify_flags(T, R, 0)
-    t = np.arange(T)
-    topk_np = np.stack([t % R, (t + 1) % R], axis=1).astype(np.int64)    # one expert per rank
     buf = ops.Buffer(T, 2, R, R, device=gu.DEV)
+    for src in range(R):
+        flags = wl.reference_notify_flags(T, R, src)
+        _, h = gu.run_fused_layout(buf, notify_topk(T, R, src), num_channels=C)
+        np.testing.assert_array_equal(h.is_token_in_rank.cpu().numpy().view(np.uint8), flags)
+        np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy(), oracle.channel_prefix(flags, C))
+
+
+@pytest.mark.parametrize("T", [7, 4096, 4097])
+@pytest.mark.parametrize("R", [2, 4, 8])
+def test_both_prefix_matrices_of_the_notify_cases_from_one_launch(oracle, T, R):
+    """notify_dispatch's two outputs (example047 .cu:112-143) from one launch with the reference's
+    channel count: the R source ranks' batches of T tokens laid end to end are R chunks of exactly
+    ceil(R T / R) = T tokens, so rank_prefix_matrix must be the harness's expected_rank_prefix
+    (.cu:352-360: counts[src, dst] summed over sources 0..src) and channel_prefix_matrix the
+    per-channel prefix of the whole batch (.cu:386-428)."""
+    C = wl.reference_notify_channels(R)
+    flags = np.concatenate([wl.reference_notify_flags(T, R, src) for src in range(R)])
+    topk_np = np.concatenate([notify_topk(T, R, src) for src in range(R)])
+    buf = ops.Buffer(R * T, 2, R, R, device=gu.DEV)
     _, h = gu.run_fused_layout(buf, topk_np, num_channels=C)
     np.testing.assert_array_equal(h.is_token_in_rank.cpu().numpy().view(np.uint8), flags)
+    counts = np.stack([wl.reference_notify_flags(T, R, src).sum(axis=0) for src in range(R)]).astype(np.int32)
+    assert (counts.sum(axis=1) == 2 * T).all()                 # two distinct destinations per token
+    got = h.rank_prefix_matrix().cpu().numpy()
+    np.testing.assert_array_equal(got, oracle.rank_prefix(counts))
+    np.testing.assert_array_equal(got[-1], h.num_tokens_per_rank.cpu().numpy())
     np.testing.assert_array_equal(h.channel_prefix_matrix.cpu().numpy(), oracle.channel_prefix(flags, C))
 
 

@@ -124,6 +124,7 @@ def test_host_twin_of_the_fused_layout(oracle, shape):
     np.testing.assert_array_equal(out["psum_rank_rows"], psum)
     np.testing.assert_array_equal(out["slot_rel"], slot_rel)
     np.testing.assert_array_equal(out["channel_prefix_matrix"], oracle.channel_prefix(flags, 2 * R))
+    np.testing.assert_array_equal(out["rank_prefix_matrix"], oracle.rank_prefix(gu.source_chunk_counts(flags, R)))
     np.testing.assert_array_equal(out["rank_slot_idx"], oracle.rank_slots(topk_np, R, E, gu.RANK_SLOT_BASE))
     want_order = oracle.route_order(topk_np, E, gu.TILE_TOKENS, fill=0)
     np.testing.assert_array_equal(out["route_order"], want_order)

@@ -27,6 +27,7 @@ class LayoutOutputs:
         self.off = torch.full((E + 1,), -3, **i32)
         self.psum = torch.full((R,), -3, **i32)
         self.channel_prefix = torch.full((R, channels), -3, **i32)
+        self.rank_prefix = torch.full((R, R), -3, **i32)
         self.slot_rel = torch.full((max(T, 1), K), -3, **i32)
         self.rank_slot_idx = torch.full((max(T, 1), K), -3, **i32)
         # entries past the last token are never written: same fill on both sides
@@ -37,7 +38,7 @@ class LayoutOutputs:
 
     def tensors(self):
         return [self.per_rank, self.per_expert, self.flags, self.off, self.psum, self.channel_prefix,
-                self.slot_rel, self.rank_slot_idx, self.route_order, self.tile_rank_counts,
+                self.rank_prefix, self.slot_rel, self.rank_slot_idx, self.route_order, self.tile_rank_counts,
                 self.copied_topk_idx, self.stats]
 
 
@@ -52,18 +53,19 @@ def run_both(lib, topk_np, R, E, align, channels):
     _lib.check(lib.mi_ep_dispatch_layout(
         topk.data_ptr(), T, K, R, E, align, channels, want.per_rank.data_ptr(), want.per_expert.data_ptr(),
         want.flags.data_ptr(), want.off.data_ptr(), want.psum.data_ptr(), want.channel_prefix.data_ptr(),
-        want.slot_rel.data_ptr(), want.rank_slot_idx.data_ptr(), gu.RANK_SLOT_BASE, want.route_order.data_ptr(),
-        want.tile_rank_counts.data_ptr(), want.copied_topk_idx.data_ptr(), want.stats.data_ptr(),
+        want.rank_prefix.data_ptr(), want.slot_rel.data_ptr(), want.rank_slot_idx.data_ptr(), gu.RANK_SLOT_BASE,
+        want.route_order.data_ptr(), want.tile_rank_counts.data_ptr(), want.copied_topk_idx.data_ptr(), want.stats.data_ptr(),
         ws.data_ptr(), ws_bytes, stream), "mi_ep_dispatch_layout")
     report = torch.zeros(1, dtype=torch.int32, device=gu.DEV)
     _lib.check(lib.mi_ep_dispatch_layout_static(
         topk.data_ptr(), T, K, R, E, align, channels, got.per_rank.data_ptr(), got.per_expert.data_ptr(),
         got.flags.data_ptr(), got.off.data_ptr(), got.psum.data_ptr(), got.channel_prefix.data_ptr(),
-        got.slot_rel.data_ptr(), got.rank_slot_idx.data_ptr(), gu.RANK_SLOT_BASE, got.route_order.data_ptr(),
-        got.tile_rank_counts.data_ptr(), got.copied_topk_idx.data_ptr(), got.stats.data_ptr(),
+        got.rank_prefix.data_ptr(), got.slot_rel.data_ptr(), got.rank_slot_idx.data_ptr(), gu.RANK_SLOT_BASE,
+        got.route_order.data_ptr(), got.tile_rank_counts.data_ptr(), got.copied_topk_idx.data_ptr(), got.stats.data_ptr(),
         report.data_ptr(), stream), "mi_ep_dispatch_layout_static")
     torch.cuda.synchronize()
     _lib.check(lib.mi_ep_workspace_status(ws.data_ptr(), stream), "workspace status")
+    _lib.check(lib.mi_ep_workspace_status(_lib.STATIC_SCRATCH, stream), "static scratch status")
     assert int(report.item()) == 0
     for a, b in zip(want.tensors(), got.tensors()):
         assert torch.equal(a, b)
@@ -99,9 +101,44 @@ def test_static_layout_refuses_shapes_beyond_its_scratch():
     # nothing is launched, so no buffer is touched: null outputs are never reached
     one = torch.zeros(8, dtype=torch.int64, device=gu.DEV)
     rc = lib.mi_ep_dispatch_layout_static(one.data_ptr(), T, K, R, E, 1, 0, one.data_ptr(), one.data_ptr(),
-                                          one.data_ptr(), None, None, None, None, None, 0, None, None, None,
+                                          one.data_ptr(), None, None, None, None, None, None, 0, None, None, None,
                                           None, None, torch.cuda.current_stream().cuda_stream)
     assert rc == E2BIG
     assert "static scratch" in _lib.strerror(rc)
     torch.cuda.synchronize()
     assert int(one.sum().item()) == 0
+
+
+def test_static_layout_reports_an_expired_wait_and_recovers(oracle):
+    """Failure handling on the library's own scratch, forced from the host: with its wait limit set to
+    one poll, launches over hundreds of tiles give up a wait of their scan; every launch still ends,
+    the caller's report word and the scratch's status both say so, and after the scratch is
+    initialised again the entry point gives the workspace entry's results."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    T, K, R, E = 65536, 8, 8, 256                    # 256 tiles x 264 columns: within the scratch
+    topk_np = wl.uniform_distinct_topk(np.random.default_rng(3), T, E, K)
+    topk = torch.from_numpy(topk_np).to(gu.DEV)
+    out = LayoutOutputs(T, K, R, E, 4, lib)
+    report = torch.zeros(1, dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.mi_ep_workspace_set_wait_limit(_lib.STATIC_SCRATCH, 1, stream), "static wait limit")
+    try:
+        expired = False
+        for _ in range(20):
+            _lib.check(lib.mi_ep_dispatch_layout_static(
+                topk.data_ptr(), T, K, R, E, 1, 4, out.per_rank.data_ptr(), out.per_expert.data_ptr(),
+                out.flags.data_ptr(), out.off.data_ptr(), out.psum.data_ptr(), out.channel_prefix.data_ptr(),
+                out.rank_prefix.data_ptr(), out.slot_rel.data_ptr(), None, 0, None, None, None, None,
+                report.data_ptr(), stream), "mi_ep_dispatch_layout_static")
+            torch.cuda.synchronize()
+            if int(report.item()) != 0:
+                expired = True
+                break
+        assert expired, "no wait expired with a one-poll limit over hundreds of tiles"
+        assert int(report.item()) == -110
+        assert lib.mi_ep_workspace_status(_lib.STATIC_SCRATCH, stream) == -110
+    finally:
+        _lib.check(lib.mi_ep_workspace_init(_lib.STATIC_SCRATCH, 0, stream), "static scratch re-init")
+    assert lib.mi_ep_workspace_status(_lib.STATIC_SCRATCH, stream) == 0
+    rng = np.random.default_rng(9)
+    run_both(lib, wl.uniform_distinct_topk(rng, 5000, 64, 4), 8, 64, 1, 16)
