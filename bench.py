@@ -48,6 +48,9 @@ def parse_args():
     ap.add_argument("--no-yardsticks", action="store_true",
                     help="skip the linear copy / read / write streams measured beside the roofline")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--jit", action="store_true",
+                    help="run on a library compiled at run time with this configuration's shapes as constants "
+                         "(commbench_amd.jit); implies --no-other-configs, whose shapes such a library refuses")
     ap.add_argument("--sustained-steps", type=int, default=3000,
                     help="back-to-back steps of each sustained-load leg, timed in windows of "
                          "--sustained-window steps (0 skips the legs)")
@@ -457,6 +460,13 @@ def main():
     cfg = wl.CONFIGS[args.config]
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    jit_shapes = None
+    if args.jit:
+        from commbench_amd import jit
+        jit_shapes = dict(num_topk=cfg.num_topk, num_experts=cfg.num_experts, num_ranks=cfg.num_ranks,
+                          row_bytes=cfg.row_bytes, hidden=cfg.hidden)
+        jit.activate(**jit_shapes)
+        args.no_other_configs = True
     wk = Workload(cfg, dev, args.rotate_x)
     T = cfg.num_tokens
 
@@ -653,6 +663,8 @@ def main():
             "num_tokens": T, "hidden": cfg.hidden, "num_experts": cfg.num_experts,
             "num_topk": cfg.num_topk, "num_ranks": cfg.num_ranks, "payload": cfg.payload,
             "source_buffers": args.rotate_x,
+            "library": "shipped (every shape a run-time argument)" if jit_shapes is None
+                       else f"compiled at run time for {jit_shapes}",
             "inputs": "commbench_amd.workloads generators (PCG64 seeded 0xC0FFEE + config id): "
                       "make_routing, make_payload, make_expert_outputs",
         },

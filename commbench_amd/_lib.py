@@ -69,6 +69,15 @@ class MiEpError(RuntimeError):
         super().__init__(f"{where} failed: {code} ({strerror(code)})")
 
 
+def bind(lib: ctypes.CDLL) -> ctypes.CDLL:
+    """Gives every entry point of include/mi_ep.h its prototype on a loaded library."""
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib
+
+
 def load() -> ctypes.CDLL:
     global _lib
     if _lib is None:
@@ -76,13 +85,15 @@ def load() -> ctypes.CDLL:
             raise ImportError(
                 f"{LIB_PATH} is missing: build it with `python -m commbench_amd.build` "
                 "(there is no CPU fallback for the HIP path)")
-        lib = ctypes.CDLL(LIB_PATH)
-        for name, (restype, argtypes) in SIGNATURES.items():
-            fn = getattr(lib, name)
-            fn.restype = restype
-            fn.argtypes = argtypes
-        _lib = lib
+        _lib = bind(ctypes.CDLL(LIB_PATH))
     return _lib
+
+
+def use(lib) -> None:
+    """Makes `lib` (a library from commbench_amd.jit, already bound) the one every later call goes
+    through; None goes back to the shipped library."""
+    global _lib
+    _lib = lib
 
 
 def strerror(code: int) -> str:

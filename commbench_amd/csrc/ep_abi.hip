@@ -26,7 +26,9 @@ inline bool routing_shape_ok(int num_tokens, int num_topk, int num_ranks, int nu
   if (num_experts <= 0 || num_experts > MI_EP_MAX_EXPERTS) return false;
   if (num_experts % num_ranks != 0) return false;
   if (static_cast<long long>(num_tokens) * num_topk >= (1LL << 30)) return false;
-  return true;
+  // A library built for fixed shapes serves those only.
+  return fixed::accepts(fixed::kTopk, num_topk) && fixed::accepts(fixed::kExperts, num_experts) &&
+         fixed::accepts(fixed::kRanks, num_ranks);
 }
 
 inline int num_tiles_for(int num_tokens) { return (num_tokens + kTileTokens - 1) / kTileTokens; }
@@ -34,7 +36,7 @@ inline int num_tiles_for(int num_tokens) { return (num_tokens + kTileTokens - 1)
 inline int status_of(hipError_t e) { return e == hipSuccess ? MI_EP_OK : static_cast<int>(e); }
 
 inline bool route_count_ok(int num_tokens, int num_topk) {
-  return num_tokens >= 0 && num_topk > 0 && num_topk <= MI_EP_MAX_TOPK &&
+  return num_tokens >= 0 && num_topk > 0 && num_topk <= MI_EP_MAX_TOPK && fixed::accepts(fixed::kTopk, num_topk) &&
          static_cast<long long>(num_tokens) * num_topk < (1LL << 30);
 }
 
@@ -340,6 +342,7 @@ int mi_ep_dispatch_strided_scales(const void* x, const float* x_scales, long lon
   if (!route_count_ok(num_tokens, num_topk)) return MI_EP_EINVAL;
   if (num_experts <= 0 || num_experts > MI_EP_MAX_EXPERTS || expert_alignment < 1) return MI_EP_EINVAL;
   if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
+  if (!fixed::accepts(fixed::kExperts, num_experts) || !fixed::accepts(fixed::kRowBytes, row_bytes)) return MI_EP_EINVAL;
   if (expert_offsets == nullptr || recv_src_map == nullptr) return MI_EP_EINVAL;
   if (capacity_rows > 0 && recv_x == nullptr) return MI_EP_EINVAL;
   if (!aligned16(x) || !aligned16(recv_x) || !aligned16(route_order)) return MI_EP_EINVAL;
@@ -419,6 +422,7 @@ int mi_ep_dispatch_ranks_strided_scales(const void* x, const float* x_scales, lo
                                         int* psum_rank_tokens, int capacity_rows, void* stream) {
   if (!routing_shape_ok(num_tokens, num_topk, num_ranks, num_experts)) return MI_EP_EINVAL;
   if (row_bytes <= 0 || row_bytes % 16 != 0 || num_scales < 0 || capacity_rows < 0) return MI_EP_EINVAL;
+  if (!fixed::accepts(fixed::kRowBytes, row_bytes)) return MI_EP_EINVAL;
   if (num_tokens_per_rank == nullptr || psum_rank_tokens == nullptr) return MI_EP_EINVAL;
   if (capacity_rows > 0 && recv_x == nullptr) return MI_EP_EINVAL;
   if (!aligned16(x) || !aligned16(recv_x)) return MI_EP_EINVAL;
@@ -526,7 +530,7 @@ int mi_ep_combine(const void* y, int num_rows, const int* slot_map, const float*
                   int flags, void* stream) {
   if (!route_count_ok(num_tokens, num_topk)) return MI_EP_EINVAL;
   if ((flags & ~MI_EP_COMBINE_STREAM_OUTPUT) != 0) return MI_EP_EINVAL;
-  if (hidden <= 0 || hidden % 8 != 0 || num_rows < 0) return MI_EP_EINVAL;
+  if (hidden <= 0 || hidden % 8 != 0 || num_rows < 0 || !fixed::accepts(fixed::kHidden, hidden)) return MI_EP_EINVAL;
   // Units of the staged schedule are counted in int: rows of a group times 16-byte vectors.
   if (static_cast<long long>(hidden) / 8 >= (1LL << 24)) return MI_EP_EINVAL;
   if (num_rows > 0 && y == nullptr) return MI_EP_EINVAL;

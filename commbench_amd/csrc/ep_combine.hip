@@ -127,8 +127,9 @@ __device__ __forceinline__ void combine_unit(const CombineArgs& a, const int tok
 }
 
 template <int kTopk, int kBatchVecs>
-__global__ __launch_bounds__(kCombineThreads) void ep_combine_kernel(const CombineArgs a,
+__global__ __launch_bounds__(kCombineThreads) void ep_combine_kernel(const CombineArgs args,
                                                                      const int batches_per_row) {
+  const CombineArgs a = fixed::apply(args);
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
   const long long unit = static_cast<long long>(blockIdx.x) * kCombineWaves + wave;
@@ -162,10 +163,11 @@ __global__ __launch_bounds__(kCombineThreads) void ep_combine_kernel(const Combi
 // groups of tokens below `through_tokens` are written through and the rest is streamed ("nt"): with the
 // share that still fits, 16384 x 8 KiB rows gain 10 us of 388 and 12288 x 14 KiB rows 9 us of 520.
 template <int kTopk, int kRegUnits>
-__global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const CombineArgs a,
+__global__ __launch_bounds__(kStagedThreads) void ep_combine_staged_kernel(const CombineArgs args,
                                                                           const int group_tokens,
                                                                           const int lds_units,
                                                                           const int through_tokens) {
+  const CombineArgs a = fixed::apply(args);
   extern __shared__ vec16 stage[];  // [lds_units][64]
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
@@ -328,21 +330,32 @@ hipError_t launch_combine_k(const CombineArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// A library built for one top-k carries that instantiation only.
+template <int kFixedTopk>
+hipError_t launch_combine_for(const CombineArgs& a, hipStream_t stream) {
+  if constexpr (kFixedTopk != 0) {
+    return launch_combine_k<kFixedTopk>(a, stream);
+  } else {
+    switch (a.num_topk) {
+      case 1: return launch_combine_k<1>(a, stream);
+      case 2: return launch_combine_k<2>(a, stream);
+      case 3: return launch_combine_k<3>(a, stream);
+      case 4: return launch_combine_k<4>(a, stream);
+      case 5: return launch_combine_k<5>(a, stream);
+      case 6: return launch_combine_k<6>(a, stream);
+      case 7: return launch_combine_k<7>(a, stream);
+      case 8: return launch_combine_k<8>(a, stream);
+      default: return hipErrorInvalidValue;
+    }
+  }
+}
+
 }  // namespace
 
-hipError_t launch_combine(const CombineArgs& a, hipStream_t stream) {
+hipError_t launch_combine(const CombineArgs& args, hipStream_t stream) {
+  const CombineArgs a = fixed::apply(args);
   if (a.num_tokens == 0) return hipSuccess;
-  switch (a.num_topk) {
-    case 1: return launch_combine_k<1>(a, stream);
-    case 2: return launch_combine_k<2>(a, stream);
-    case 3: return launch_combine_k<3>(a, stream);
-    case 4: return launch_combine_k<4>(a, stream);
-    case 5: return launch_combine_k<5>(a, stream);
-    case 6: return launch_combine_k<6>(a, stream);
-    case 7: return launch_combine_k<7>(a, stream);
-    case 8: return launch_combine_k<8>(a, stream);
-    default: return hipErrorInvalidValue;
-  }
+  return launch_combine_for<fixed::kTopk>(a, stream);
 }
 
 }  // namespace mi_ep

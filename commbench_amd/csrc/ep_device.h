@@ -200,6 +200,79 @@ hipError_t launch_copy_yardstick(vec16* dst, const vec16* src, size_t vecs, hipS
 hipError_t launch_read_yardstick(const vec16* src, size_t vecs, uint32_t* sink, hipStream_t stream);
 hipError_t launch_write_yardstick(vec16* dst, size_t vecs, hipStream_t stream);
 
+// ---- shapes fixed at build time: the plug-in point for run-time compilation ---------------
+// The reference compiles its dispatch and combine kernels per shape: top-k, experts, ranks and the
+// hidden size are template parameters filled in by a just-in-time build of one overlaid header
+// (example080 .cu:17-30; its harness, build_and_run.py:154-172,678).  The shipped library takes
+// every shape at run time; the same sources built with any of the macros below fold that shape
+// into the kernels as a constant and refuse calls with another (MI_EP_EINVAL).  0 = not fixed.
+#ifndef MI_EP_FIXED_TOPK
+#define MI_EP_FIXED_TOPK 0
+#endif
+#ifndef MI_EP_FIXED_EXPERTS
+#define MI_EP_FIXED_EXPERTS 0
+#endif
+#ifndef MI_EP_FIXED_RANKS
+#define MI_EP_FIXED_RANKS 0
+#endif
+#ifndef MI_EP_FIXED_ROW_BYTES  // bytes of a dispatch payload row
+#define MI_EP_FIXED_ROW_BYTES 0
+#endif
+#ifndef MI_EP_FIXED_HIDDEN  // bf16 elements of a combine row
+#define MI_EP_FIXED_HIDDEN 0
+#endif
+namespace fixed {
+constexpr int kTopk = MI_EP_FIXED_TOPK, kExperts = MI_EP_FIXED_EXPERTS, kRanks = MI_EP_FIXED_RANKS;
+constexpr int kRowBytes = MI_EP_FIXED_ROW_BYTES, kHidden = MI_EP_FIXED_HIDDEN;
+static_assert(kTopk >= 0 && kTopk <= kMaxTopk && kRanks >= 0 && kRanks <= kMaxRanks && kExperts >= 0 &&
+                  kExperts <= kMaxExperts && kRowBytes % 16 == 0 && kHidden % 8 == 0,
+              "fixed shapes out of range");
+static_assert(kRanks == 0 || kExperts % kRanks == 0, "fixed experts must be divisible by fixed ranks");
+
+constexpr bool accepts(int fixed_value, long long given) { return fixed_value == 0 || given == fixed_value; }
+
+// The arguments with every fixed shape replaced by its constant (the identity in the shipped
+// library): kernels start from this copy, so that the compiler sees the constants.
+__host__ __device__ inline LayoutArgs apply(LayoutArgs a) {
+  if (kTopk != 0) {
+    a.num_topk = kTopk;
+    a.inv_topk = ((1u << 19) + kTopk - 1) / (kTopk != 0 ? kTopk : 1);
+  }
+  if (kRanks != 0) a.num_ranks = kRanks;
+  if (kExperts != 0) {
+    a.num_experts = kExperts;
+    int bits = 1;
+    while ((1 << bits) < kExperts) ++bits;
+    a.expert_bits = bits;
+  }
+  if (kExperts != 0 && kRanks != 0) {
+    constexpr int per_rank = kRanks != 0 ? kExperts / kRanks : 1;
+    a.experts_per_rank = per_rank;
+    a.inv_experts_per_rank = ((1u << 22) + per_rank - 1) / (per_rank != 0 ? per_rank : 1);
+  }
+  return a;
+}
+__host__ __device__ inline PermuteArgs apply(PermuteArgs a) {
+  if (kTopk != 0) a.num_topk = kTopk;
+  if (kExperts != 0) a.num_experts = kExperts;
+  if (kRowBytes != 0) a.row_vecs = kRowBytes / 16;
+  return a;
+}
+__host__ __device__ inline RankPermuteArgs apply(RankPermuteArgs a) {
+  if (kTopk != 0) a.num_topk = kTopk;
+  if (kExperts != 0) a.num_experts = kExperts;
+  if (kRanks != 0) a.num_ranks = kRanks;
+  if (kExperts != 0 && kRanks != 0) a.experts_per_rank = kExperts / (kRanks != 0 ? kRanks : 1);
+  if (kRowBytes != 0) a.row_vecs = kRowBytes / 16;
+  return a;
+}
+__host__ __device__ inline CombineArgs apply(CombineArgs a) {
+  if (kTopk != 0) a.num_topk = kTopk;
+  if (kHidden != 0) a.row_vecs = kHidden / 8;
+  return a;
+}
+}  // namespace fixed
+
 // ---- device helpers -------------------------------------------------------
 #ifdef __HIPCC__
 __device__ __forceinline__ int lane_id() { return static_cast<int>(threadIdx.x) & (kWave - 1); }

@@ -88,7 +88,8 @@ __device__ __forceinline__ void store_token_flags(uint8_t* is_token_in_rank, int
   }
 }
 
-__global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const LayoutArgs a) {
+__global__ __launch_bounds__(kLayoutThreads) void ep_layout_fused_kernel(const LayoutArgs args) {
+  const LayoutArgs a = fixed::apply(args);
   extern __shared__ int smem[];
   const int E = a.num_experts, R = a.num_ranks, K = a.num_topk, T = a.num_tokens;
   const int cols = E + R;
@@ -721,7 +722,8 @@ hipError_t launch_fill_u32(uint32_t* dst, size_t count, uint32_t value, hipStrea
   return hipGetLastError();
 }
 
-hipError_t launch_layout_fused(const LayoutArgs& a, hipStream_t stream) {
+hipError_t launch_layout_fused(const LayoutArgs& args, hipStream_t stream) {
+  const LayoutArgs a = fixed::apply(args);
   static_assert(kMaxExperts <= kLayoutThreads, "the offset scan takes one expert per thread");
   const int E = a.num_experts;
   const int cols = E + a.num_ranks;

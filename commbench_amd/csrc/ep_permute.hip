@@ -85,8 +85,9 @@ __device__ __forceinline__ void write_pad_markers(const PermuteArgs& a, const lo
 }
 
 template <int kBatchVecs, bool kStreamStores>
-__global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteArgs a,
+__global__ __launch_bounds__(kPushThreads) void ep_permute_kernel(const PermuteArgs args,
                                                                   const int batches_per_row) {
+  const PermuteArgs a = fixed::apply(args);
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
   const long long unit = static_cast<long long>(blockIdx.x) * kPushWaves + wave;
@@ -211,10 +212,11 @@ __device__ __forceinline__ void pad_markers_from_prefetch_workgroup(const Permut
 // each take kVecs KiB-per-wave parts of it: no idle lanes on rows that are not a multiple of the
 // part size (kVecs is 1 then and there is one part).
 template <int kVecs, bool kPads, bool kZeroPads, bool kScales, bool kRowWide>
-__global__ __launch_bounds__(kRowWide ? static_cast<int>(kRowWideBytesMax / sizeof(vec16)) : kPushThreads) void ep_permute_tiles_kernel(const PermuteArgs a,
+__global__ __launch_bounds__(kRowWide ? static_cast<int>(kRowWideBytesMax / sizeof(vec16)) : kPushThreads) void ep_permute_tiles_kernel(const PermuteArgs args,
                                                                                          const int num_tiles,
                                                                                          const int pad_items_per_tile) {
   static_assert(!kRowWide || kVecs == 1, "a row-wide workgroup moves one vector per lane");
+  const PermuteArgs a = fixed::apply(args);
   constexpr int prefetch_ys = kPrefetchGroups;
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
@@ -392,8 +394,9 @@ hipError_t launch_permute_tiles(const PermuteArgs& a, const dim3 grid, const int
 // example081 .cu:22-60).  Same wave-per-(token, KiB) shape as ep_permute_kernel; a token's
 // destinations are the first slot of each distinct rank, whose position inside the rank's rows
 // the layout kernel has already fixed (rank_slot_idx).
-__global__ __launch_bounds__(kPushThreads) void ep_permute_ranks_kernel(const RankPermuteArgs a,
+__global__ __launch_bounds__(kPushThreads) void ep_permute_ranks_kernel(const RankPermuteArgs args,
                                                                        const int batches_per_row) {
+  const RankPermuteArgs a = fixed::apply(args);
   const int lane = lane_id();
   const int wave = static_cast<int>(threadIdx.x) >> 6;
   const long long unit = static_cast<long long>(blockIdx.x) * kPushWaves + wave;
@@ -684,7 +687,8 @@ bool destination_order_pays(const PermuteArgs& a, const DeviceTraits& dev) {
   return kTileTokens * a.num_topk >= kRunRowsMin * a.num_experts;  // expected rows per (tile, expert)
 }
 
-hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream) {
+hipError_t launch_permute(const PermuteArgs& args, int schedule, hipStream_t stream) {
+  const PermuteArgs a = fixed::apply(args);
   const long long pad_items = a.expert_alignment > 1 ? static_cast<long long>(a.num_experts) * (a.expert_alignment - 1) : 0;
   if (a.num_tokens == 0 && pad_items == 0) return hipSuccess;
   bool by_destination = a.num_tokens > 0 && a.route_order != nullptr && schedule == kPermuteByDestination;
@@ -731,7 +735,8 @@ hipError_t launch_permute(const PermuteArgs& a, int schedule, hipStream_t stream
   return hipGetLastError();
 }
 
-hipError_t launch_permute_ranks(const RankPermuteArgs& a, hipStream_t stream) {
+hipError_t launch_permute_ranks(const RankPermuteArgs& args, hipStream_t stream) {
+  const RankPermuteArgs a = fixed::apply(args);
   const int batches = (a.row_vecs + kWave - 1) / kWave;
   // At least one unit, so that the per-rank row totals are written for an empty batch too.
   const long long units = a.num_tokens > 0 ? static_cast<long long>(a.num_tokens) * batches : 1;
