@@ -142,3 +142,62 @@ def test_static_layout_reports_an_expired_wait_and_recovers(oracle):
     assert lib.mi_ep_workspace_status(_lib.STATIC_SCRATCH, stream) == 0
     rng = np.random.default_rng(9)
     run_both(lib, wl.uniform_distinct_topk(rng, 5000, 64, 4), 8, 64, 1, 16)
+
+
+def test_static_layout_replays_in_a_graph(oracle):
+    """What the entry point is for: captured in a HIP graph (no allocation, no memset node, the scratch
+    address resolved by an eager call beforehand), every replay must give the eager result for the
+    inputs of the moment, with eager work and synchronisations between the replays."""
+    lib = _lib.load()
+    T, K, R, E = 5000, 8, 8, 256                      # 20 tiles: static tiles, gathered scan
+    topk = torch.empty((T, K), dtype=torch.int64, device=gu.DEV)
+    out = LayoutOutputs(T, K, R, E, 16, lib)
+    report = torch.zeros(1, dtype=torch.int32, device=gu.DEV)
+
+    def launch(stream):
+        _lib.check(lib.mi_ep_dispatch_layout_static(
+            topk.data_ptr(), T, K, R, E, 4, 16, out.per_rank.data_ptr(), out.per_expert.data_ptr(),
+            out.flags.data_ptr(), out.off.data_ptr(), out.psum.data_ptr(), out.channel_prefix.data_ptr(),
+            out.rank_prefix.data_ptr(), out.slot_rel.data_ptr(), out.rank_slot_idx.data_ptr(), gu.RANK_SLOT_BASE,
+            out.route_order.data_ptr(), out.tile_rank_counts.data_ptr(), None, None, report.data_ptr(), stream),
+            "mi_ep_dispatch_layout_static")
+
+    def load_inputs(seed):
+        rng = np.random.default_rng(seed)
+        t = wl.zipf_distinct_topk(rng, T, E, K, 1.2)
+        t[rng.random((T, K)) < 0.05] = -1
+        topk.copy_(torch.from_numpy(t))
+        return t
+
+    load_inputs(0)
+    launch(torch.cuda.current_stream().cuda_stream)          # eager: resolves the scratch's address
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for seed in (1, 2, 3):
+        t_np = load_inputs(seed)
+        for t in out.tensors()[:-2]:                         # eager work between the replays
+            t.view(torch.uint8).fill_(0x5A)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(report.item()) == 0
+        per_rank, per_expert, flags = oracle.layout(t_np, R, E)
+        off, psum = oracle.expert_offsets(per_expert, R, 4)
+        slot_rel, _, _, _ = oracle.slot_maps(t_np, E, off)
+        np.testing.assert_array_equal(out.per_rank.cpu().numpy(), per_rank)
+        np.testing.assert_array_equal(out.per_expert.cpu().numpy(), per_expert)
+        np.testing.assert_array_equal(out.flags.cpu().numpy()[:T], flags)
+        np.testing.assert_array_equal(out.off.cpu().numpy(), off)
+        np.testing.assert_array_equal(out.psum.cpu().numpy(), psum)
+        np.testing.assert_array_equal(out.slot_rel.cpu().numpy(), slot_rel)
+        np.testing.assert_array_equal(out.channel_prefix.cpu().numpy(), oracle.channel_prefix(flags, 16))
+        np.testing.assert_array_equal(out.rank_prefix.cpu().numpy(),
+                                      oracle.rank_prefix(gu.source_chunk_counts(flags, R)))
+        np.testing.assert_array_equal(out.rank_slot_idx.cpu().numpy(),
+                                      oracle.rank_slots(t_np, R, E, gu.RANK_SLOT_BASE))
+    assert lib.mi_ep_workspace_status(_lib.STATIC_SCRATCH, torch.cuda.current_stream().cuda_stream) == 0
