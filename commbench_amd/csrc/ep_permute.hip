@@ -716,11 +716,14 @@ hipError_t launch_permute(const PermuteArgs& args, int schedule, hipStream_t str
       pad_items_per_tile = static_cast<int>((pad_items + tiles - 1) / tiles);
       ys += (pad_items_per_tile + parts - 1) / parts;
     }
-    if (rounds > 65535 || ys > 65535 || parts * kDies > 65535) return hipErrorInvalidValue;
-    const dim3 grid(static_cast<unsigned>(parts * kDies), static_cast<unsigned>(ys), static_cast<unsigned>(rounds));
-    if (row_wide)
-      return launch_permute_tiles<1, true>(a, grid, (a.row_vecs + kWave - 1) / kWave * kWave, tiles, pad_items_per_tile, stream);
-    return launch_permute_tiles<1, false>(a, grid, kPushThreads, tiles, pad_items_per_tile, stream);
+    // A grid that does not fit the launch limits (over 16 million tokens, or millions of pad rows to
+    // zero per tile) is left to the token-order kernel below: the outputs are the same.
+    if (rounds <= 65535 && ys <= 65535 && parts * kDies <= 65535) {
+      const dim3 grid(static_cast<unsigned>(parts * kDies), static_cast<unsigned>(ys), static_cast<unsigned>(rounds));
+      if (row_wide)
+        return launch_permute_tiles<1, true>(a, grid, (a.row_vecs + kWave - 1) / kWave * kWave, tiles, pad_items_per_tile, stream);
+      return launch_permute_tiles<1, false>(a, grid, kPushThreads, tiles, pad_items_per_tile, stream);
+    }
   }
   const int batches = (a.row_vecs + kWave - 1) / kWave;
   long long units = static_cast<long long>(a.num_tokens) * batches;

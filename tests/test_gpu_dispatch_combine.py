@@ -117,6 +117,19 @@ def test_alignment_pads_are_zero_rows(oracle, align):
     assert pads.any() and not gu.as_bytes(recv_x)[:off[-1]][pads].any()
 
 
+def test_huge_alignment_beyond_the_destination_order_grid(oracle):
+    """An alignment so large that the zeroed pad rows of a tile no longer fit the destination-order
+    kernel's grid (65535 list entries per tile): the call must fall back to the token-order kernel by
+    itself, with the same outputs, under either schedule flag."""
+    rng = np.random.default_rng(41)
+    T, K, E, R, H, align = 300, 2, 8, 2, 8, 40000                 # 16-byte rows, 320 000 possible pad rows
+    topk_np = wl.uniform_distinct_topk(rng, T, E, K)
+    w_np = wl.softmax_gates(rng, T, K)
+    x_cpu = wl.bf16_normal(rng, T, H)
+    recv_x, h, ref = dispatch_and_check(oracle, (E, R), topk_np, w_np, x_cpu, None, align=align)
+    assert int(ref["expert_offsets"][-1]) == E * align and (ref["recv_src_map"] < 0).sum() == E * align - T * K
+
+
 @pytest.mark.parametrize("schedule", gu.SCHEDULES)
 def test_scale_factors_through_strides(oracle, schedule):
     """Scale factors in a column-major, padded tensor on the way in and column-major on the way out
