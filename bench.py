@@ -7,7 +7,8 @@ bf16 expert outputs.  Inputs come from the same seeded generators the parity tes
 (commbench_amd/workloads.py).  Prints one JSON line (see the keys below).  The CPU checker is
 timed on the same workload and inputs as a reported baseline.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config target|c2|c3|c4|c5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config target|c2|c3|c4|c5] [--jit]
+                    [--sustained-steps N --sustained-window M]
 """
 import argparse
 import hashlib
