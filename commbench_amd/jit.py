@@ -103,7 +103,7 @@ def compile_library(**shapes: int) -> str:
         return out
     os.makedirs(cache_dir(), exist_ok=True)
     # The sources include "../../include/mi_ep.h": stage them in a tree of the same shape.
-    stage = out[:-3] + "_src"
+    stage = out[:-3] + f"_src{os.getpid()}"          # per process: two may build the same library at once
     shutil.rmtree(stage, ignore_errors=True)
     csrc = os.path.join(stage, "commbench_amd", "csrc")
     os.makedirs(csrc)
@@ -112,12 +112,12 @@ def compile_library(**shapes: int) -> str:
     for name, path in source_files().items():
         shutil.copy(path, os.path.join(csrc, name))
     cmd = [_hipcc(), *hip_build.HIPCC_FLAGS, *[f"-D{k}={v}" for k, v in _defines(shapes).items()],
-           "-o", out + ".tmp"] + [os.path.join(csrc, s) for s in hip_build.SOURCES]
+           "-o", f"{out}.{os.getpid()}.tmp"] + [os.path.join(csrc, s) for s in hip_build.SOURCES]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     shutil.rmtree(stage, ignore_errors=True)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + proc.stdout + proc.stderr)
-    os.replace(out + ".tmp", out)
+    os.replace(f"{out}.{os.getpid()}.tmp", out)     # atomic: a reader sees the old file or the whole new one
     return out
 
 
